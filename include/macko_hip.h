@@ -1,0 +1,93 @@
+/*
+ * macko_hip.h -- C ABI of libmacko_hip.so: MACKO fp16 sparse matrix-vector product and
+ * compressor for AMD gfx950 (MI355X).
+ *
+ * Plain pointers and sizes only.  Every pointer is a DEVICE pointer unless said otherwise.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).  No entry point
+ * allocates, frees or keeps caller-visible memory; nothing synchronises unless said otherwise.
+ * Return value: 0 on success, a positive hipError_t from the HIP runtime, or one of the
+ * negative MACKO_E_* codes below.  macko_hip_error_string() explains either kind.
+ *
+ * Compressed matrix ("the 5-tuple" of the upstream Python API, src/macko_spmv/__init__.py:120-131):
+ *   values   fp16  [P]      stored entries (non-zeros and padding entries), P a multiple of 8
+ *   deltas   uint8 [P/2]    4-bit column gaps, entry j in byte j/2, low nibble when j is even
+ *   row_ptr  int32 [rows+1] entry index where each row starts; row_ptr[rows] = n <= P < n + 8
+ *   rows, cols
+ * Column of the k-th entry of a row = (sum of the nibbles of its entries 0..k) + k.
+ */
+#ifndef MACKO_HIP_H
+#define MACKO_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MACKO_E_INVALID_ARGUMENT (-1) /* null pointer, negative size, rows*cols >= 2^31 ... */
+#define MACKO_E_NO_DEVICE (-2)        /* no usable HIP device */
+
+/* ABI version of this header (bumped on incompatible change). */
+int macko_hip_abi_version(void);
+
+/* Human-readable text for a return code of this library.  Never NULL; static storage. */
+const char *macko_hip_error_string(int code);
+
+/*
+ * y[r] = fp16( sum_k fp32(values[k]) * fp32(x[col_k]) ) for every row r, fp32 accumulation.
+ *
+ * Replaces the kernel launch in macko_spmv_launcher
+ * (src/macko_spmv/cuda/kernels_torch_launchers.cuh:15-45, kernel src/macko_spmv/cuda/kernels.cuh:34-124,
+ * alpha = 1, beta ignored).  Asynchronous on `stream`; safe to capture in a HIP graph.
+ *
+ *   padded_entries = P = number of fp16 elements in `values` (0 allowed: y is zero-filled)
+ *   x   fp16 [>= cols], 2-byte aligned (16-byte alignment is faster)
+ *   y   fp16 [rows], written for every row
+ */
+int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_ptr,
+                   const void *x, void *y, int32_t rows, int32_t cols,
+                   int64_t padded_entries, void *stream);
+
+/*
+ * y[r] = fp16( alpha * (M x)[r] + beta * fp32(y[r]) ).
+ *
+ * Replaces the macko_spmv<true> instantiation that the upstream C benchmark launches
+ * (src/macko_spmv/cuda/kernels.cuh:113-118, c_benchmarking/benchmark.cu:92-105).
+ */
+int macko_spmv_f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+                         const void *x, void *y, int32_t rows, int32_t cols,
+                         int64_t padded_entries, float alpha, float beta, void *stream);
+
+/*
+ * Compressor, step 1 of 2.  Reads the dense row-major fp16 matrix `dense` [rows, cols] and
+ * writes row_ptr[0..rows] (int32, device).  Asynchronous.  The caller then reads
+ * n = row_ptr[rows] back (one 4-byte copy + stream sync), sizes values/deltas to
+ * P = ceil(n/8)*8 and calls step 2.
+ *
+ * Steps 1+2 together replace compress_rows_cpu (src/macko_spmv/cuda/cpu_compressor.cuh:6-73)
+ * and emit bit-identical arrays.
+ */
+int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols,
+                             int32_t *row_ptr, void *stream);
+
+/*
+ * Compressor, step 2 of 2.  Fills values [P] and deltas [P/2] (both fully written, tail
+ * zero-filled) from `dense` and the row_ptr produced by step 1.  Asynchronous.
+ */
+int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
+                            const int32_t *row_ptr, void *values, void *deltas,
+                            int64_t padded_entries, void *stream);
+
+/*
+ * Inverse of the compressor: writes the dense row-major fp16 matrix [rows, cols] (every
+ * element written).  Uses the decode rule of the multiply kernel
+ * (src/macko_spmv/cuda/kernels.cuh:97-103); the upstream package has no such function, it is
+ * provided for round-trip checks at sizes a CPU decode cannot reach.
+ */
+int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr,
+                         int32_t rows, int32_t cols, void *dense, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MACKO_HIP_H */

@@ -1,0 +1,11 @@
+"""`import macko_spmv` alias of macko_spmv_amd, so code written against the upstream package
+(src/macko_spmv/__init__.py) runs unchanged on MI355X."""
+from macko_spmv_amd import (  # noqa: F401
+    LIB_NAME,
+    __version__,
+    compress,
+    decompress,
+    move_to_device,
+    multiply,
+    multiply_axpby,
+)

@@ -1,0 +1,126 @@
+"""MACKO sparse matrix-vector multiplication for AMD MI355X (gfx950).
+
+Drop-in for the Python surface of the upstream `macko_spmv` package
+(src/macko_spmv/__init__.py:110-149):
+
+    compressed = compress(M)             # 5-tuple (values, deltas, row_indices, rows, cols)
+    y = multiply(compressed, V)          # fp16 [rows]
+    compressed = move_to_device(compressed, "cuda")
+
+`multiply` goes through the torch operator `torch.ops.macko_spmv.multiply` (same schema as
+upstream, fake-tensor implementation registered, usable under torch.compile).  Both functions
+run hand-written HIP kernels through the C ABI in include/macko_hip.h; there is no CPU
+implementation, and importing this package fails if the native libraries cannot be loaded.
+"""
+import ctypes
+import os
+import types
+
+import torch
+
+from . import _build
+
+__version__ = "0.2.0"
+LIB_NAME = "macko_spmv"
+
+
+def _load_native():
+    hip_path, torch_path = _build.lib_paths()
+    if not (os.path.exists(hip_path) and os.path.exists(torch_path)):
+        # first use: compile in place, like the upstream package's JIT step at import
+        # (src/macko_spmv/__init__.py:14-102)
+        _build.build_all()
+    try:
+        hip = ctypes.CDLL(hip_path, mode=ctypes.RTLD_GLOBAL)
+        torch.ops.load_library(torch_path)
+    except OSError as exc:  # no silent fallback: the HIP path is the only path
+        raise ImportError(
+            f"macko_spmv_amd: cannot load its native libraries ({hip_path}, {torch_path}): {exc}. "
+            "Rebuild them with `python -m macko_spmv_amd._build`."
+        ) from exc
+    return hip, hip_path, torch_path
+
+
+_hip_lib, HIP_LIBRARY_PATH, TORCH_LIBRARY_PATH = _load_native()
+
+
+@torch.library.register_fake("macko_spmv::multiply")
+def _multiply_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
+    # upstream fake implementation: src/macko_spmv/__init__.py:105-107
+    return torch.empty((M_rows,), device=M_values.device, dtype=M_values.dtype)
+
+
+@torch.library.register_fake("macko_spmv::multiply_axpby")
+def _multiply_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C, alpha, beta):
+    return None
+
+
+@torch.library.register_fake("macko_spmv::decompress")
+def _decompress_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols):
+    return torch.empty((M_rows, M_cols), device=M_values.device, dtype=M_values.dtype)
+
+
+def move_to_device(compressed, device):
+    """Move the three tensors of a compressed matrix (src/macko_spmv/__init__.py:110-117)."""
+    return (
+        compressed[0].to(device=device),
+        compressed[1].to(device=device),
+        compressed[2].to(device=device),
+        compressed[3],
+        compressed[4],
+    )
+
+
+def compress(M):
+    """Dense fp16 matrix -> (values fp16[P], deltas uint8[P/2], row_indices int32[R+1], R, C).
+
+    Same routing as upstream (src/macko_spmv/__init__.py:120-131): a GPU tensor yields GPU
+    tensors, a CPU tensor yields CPU tensors, other devices raise NotImplementedError.  In both
+    supported cases the arrays are produced by the HIP compressor (a CPU tensor is staged
+    through the current GPU).
+    """
+    assert M.is_contiguous()
+    if M.device.type in ("cuda", "cpu"):
+        return tuple(torch.ops.macko_spmv.compress.default(M))
+    raise NotImplementedError()
+
+
+def multiply(compressed_M, V):
+    """y = M @ V for a compressed M; fp16 in, fp32 accumulation, fp16 out
+    (src/macko_spmv/__init__.py:134-149)."""
+    assert compressed_M[0].is_cuda
+    assert compressed_M[1].is_cuda
+    assert compressed_M[2].is_cuda
+    assert V.is_cuda
+    assert V.is_contiguous()
+    return torch.ops.macko_spmv.multiply.default(
+        compressed_M[0],
+        compressed_M[1],
+        compressed_M[2],
+        compressed_M[3],
+        compressed_M[4],
+        V,
+    )
+
+
+def multiply_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):
+    """In place C = alpha * (M @ V) + beta * C: the epilogue of the upstream kernel's
+    reuse_value_from_c instantiation (src/macko_spmv/cuda/kernels.cuh:113-118)."""
+    assert compressed_M[0].is_cuda and V.is_cuda and C.is_cuda
+    assert V.is_contiguous() and C.is_contiguous()
+    torch.ops.macko_spmv.multiply_axpby.default(
+        compressed_M[0], compressed_M[1], compressed_M[2], compressed_M[3], compressed_M[4], V, C,
+        float(alpha), float(beta),
+    )
+    return C
+
+
+def decompress(compressed_M):
+    """Dense fp16 matrix back from a compressed one (GPU tensors).  Not part of the upstream API."""
+    assert compressed_M[0].is_cuda
+    return torch.ops.macko_spmv.decompress.default(*compressed_M[:5])
+
+
+# Names some upstream callers reach for (src/macko_spmv/__init__.py:36,90,141).
+__compressor_lib = types.SimpleNamespace(cpu_compress=lambda M: tuple(torch.ops.macko_spmv.compress.default(M)))
+__multiply_lib = types.SimpleNamespace(macko_spmv_launcher=torch.ops.macko_spmv.multiply.default)

@@ -1,0 +1,107 @@
+"""Build recipes for the two native libraries of this package.
+
+  libmacko_hip.so    torch-free HIP kernels behind the C ABI of include/macko_hip.h (gfx950)
+  libmacko_torch.so  PyTorch-ROCm operator library that forwards to the C ABI
+
+Both are built in-tree (next to this file) unless MACKO_SPMV_BUILD_DIRECTORY names another
+directory -- the same variable the upstream package reads for its JIT cache
+(src/macko_spmv/__init__.py:12).  hipcc cross-compiles for gfx950 without a GPU present.
+
+Run `python -m macko_spmv_amd._build` to (re)build both.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_PKG)
+_CSRC = os.path.join(_PKG, "csrc")
+_INCLUDE = os.path.join(_ROOT, "include")
+
+HIP_LIB = "libmacko_hip.so"
+TORCH_LIB = "libmacko_torch.so"
+ARCH = "gfx950"
+
+HIP_SOURCES = ["macko_spmv.hip", "macko_compress.hip", "macko_runtime.hip"]
+TORCH_SOURCES = ["macko_torch.cpp"]
+
+
+def build_directory():
+    d = os.environ.get("MACKO_SPMV_BUILD_DIRECTORY", "")
+    if d:
+        os.makedirs(d, exist_ok=True)
+        return d
+    return _PKG
+
+
+def lib_paths():
+    d = build_directory()
+    return os.path.join(d, HIP_LIB), os.path.join(d, TORCH_LIB)
+
+
+def _hipcc():
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found: a ROCm toolchain is required to build macko_spmv_amd")
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed:\n" + " ".join(cmd) + "\n" + proc.stdout)
+    if verbose and proc.stdout.strip():
+        print(proc.stdout, flush=True)
+
+
+def build_hip(verbose=False):
+    out, _ = lib_paths()
+    cmd = [
+        _hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+        # keep the compiler from forming packed fp32 VALU ops (device pass; the host pass ignores it)
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Wno-unused-command-line-argument",
+        f"-I{_INCLUDE}", f"-I{_CSRC}",
+        *[os.path.join(_CSRC, s) for s in HIP_SOURCES],
+        "-o", out,
+    ]
+    _run(cmd, verbose)
+    return out
+
+
+def build_torch(verbose=False):
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    hip_lib, out = lib_paths()
+    if not os.path.exists(hip_lib):
+        build_hip(verbose)
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = [
+        _hipcc(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+        "-Wno-unused-command-line-argument",
+        f"-I{_INCLUDE}",
+        *[f"-I{p}" for p in ce.include_paths("cuda")],
+        *[os.path.join(_CSRC, s) for s in TORCH_SOURCES],
+        "-x", "none",
+        *[f"-L{p}" for p in ce.library_paths("cuda") if os.path.isdir(p)],
+        f"-L{os.path.dirname(hip_lib)}",
+        "-lmacko_hip", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-lamdhip64",
+        "-Wl,-rpath,$ORIGIN",
+        "-o", out,
+    ]
+    _run(cmd, verbose)
+    return out
+
+
+def build_all(verbose=False):
+    return build_hip(verbose), build_torch(verbose)
+
+
+if __name__ == "__main__":
+    for path in build_all(verbose="-q" not in sys.argv):
+        print("built", path)

@@ -1,0 +1,304 @@
+// MACKO fp16 compressor and decompressor for gfx950 (wave64).
+//
+// The format is restated from src/macko_spmv/cuda/cpu_compressor.cuh:6-73 of the upstream
+// package as a per-column rule that needs no sequential walk:
+//   column x of a row stores an entry when its element is non-zero as a float (so -0.0 does
+//   not count and NaN does), or when x - p is a positive multiple of 16, p being the column
+//   of the previous non-zero (-1 before the first) -- a padding entry.  The nibble of a
+//   non-zero is (x - p - 1) & 15, of a padding entry 15.  Entries after the row's last
+//   non-zero are not stored.  A stored element keeps its bits (a padding entry keeps the sign
+//   of its zero); a NaN is stored as 0x7fff, the result of CUDA's float->half conversion that
+//   the upstream code routes every value through.
+//
+// Pass 1 (count_rows_kernel + scan_rows_kernel) produces row_ptr; pass 2 (fill_rows_kernel)
+// writes values and nibbles.  One wave owns one row in both passes; lanes take 8 consecutive
+// columns and learn the previous non-zero's column from a DPP running maximum.
+
+#include "macko_common.h"
+
+namespace macko {
+namespace {
+
+constexpr int kRowsPerBlock = 4;              // waves per workgroup, one row each
+constexpr int kBlock = kRowsPerBlock * kWave;
+constexpr int kNoColumn = (int)0x80000000;
+
+// 8 consecutive fp16 elements of a row, zero beyond `cols`.
+__device__ __forceinline__ u32x4 load8(const uint16_t *__restrict__ row, int col, int cols, bool vector_ok)
+{
+    u32x4 v = {0, 0, 0, 0};
+    if (col + 8 <= cols && vector_ok) {
+        v = *reinterpret_cast<const u32x4 *>(row + col);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            u32 h = (col + i < cols) ? row[col + i] : 0u;
+            v[i >> 1] |= h << (16 * (i & 1));
+        }
+    }
+    return v;
+}
+
+__device__ __forceinline__ u32 half_at(const u32x4 &v, int i)
+{
+    return (v[i >> 1] >> (16 * (i & 1))) & 0xffffu;
+}
+
+// bit i set when element i is non-zero as a float
+__device__ __forceinline__ u32 nonzero_bits(const u32x4 &v)
+{
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m |= ((half_at(v, i) & 0x7fffu) != 0 ? 1u : 0u) << i;
+    return m;
+}
+
+// Column of the last non-zero strictly before this lane's chunk, given the lane's own last
+// non-zero column (kNoColumn if none) and the carry from earlier passes.  Also returns the
+// last non-zero column of the whole pass through `pass_last`.
+__device__ __forceinline__ int previous_nonzero(int own_last, int carry, int lane, int &pass_last)
+{
+    const int incl = wave_scan_max_inclusive(own_last);
+    pass_last = __builtin_amdgcn_readlane(incl, kWave - 1);
+    int before = __shfl_up(incl, 1);
+    before = lane == 0 ? kNoColumn : before;
+    return before > carry ? before : carry;
+}
+
+__device__ __forceinline__ int wave_sum_int(int x)
+{
+    return __builtin_amdgcn_readlane(wave_scan_inclusive(x), kWave - 1);
+}
+
+__global__ void __launch_bounds__(kBlock) count_rows_kernel(const uint16_t *__restrict__ dense, int rows,
+                                                            int cols, int *__restrict__ counts)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + uniform(threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint16_t *src = dense + (size_t)row * (size_t)cols;
+    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+    int carry = -1;  // column of the last non-zero seen in earlier passes
+    int mine = 0;
+    for (int c0 = 0; c0 < cols; c0 += kTile) {
+        const int col = c0 + lane * kChunk;
+        const u32x4 v = load8(src, col, cols, vector_ok && col < cols);
+        const u32 nz = nonzero_bits(v);
+        const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
+        int pass_last;
+        int p = previous_nonzero(own_last, carry, lane, pass_last);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (nz & (1u << i)) {
+                mine += 1 + ((col + i - p - 1) >> 4);
+                p = col + i;
+            }
+        }
+        carry = pass_last > carry ? pass_last : carry;
+    }
+    const int total = wave_sum_int(mine);
+    if (lane == 0) counts[row] = total;
+}
+
+// row_ptr[0] = 0, row_ptr[r+1] = counts[0] + ... + counts[r].  `counts` aliases row_ptr + 1.
+// One workgroup; each thread owns a contiguous slice.
+__global__ void __launch_bounds__(1024) scan_rows_kernel(int *__restrict__ row_ptr, int rows)
+{
+    __shared__ int wave_totals[16];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid >> 6;
+    const int per = (rows + 1023) / 1024;
+    const int begin = tid * per < rows ? tid * per : rows;
+    const int end = begin + per < rows ? begin + per : rows;
+    int *counts = row_ptr + 1;
+    int sum = 0;
+    for (int i = begin; i < end; ++i) sum += counts[i];
+    const int incl = wave_scan_inclusive(sum);
+    if (lane == kWave - 1) wave_totals[wave] = incl;
+    __syncthreads();
+    int base = incl - sum;
+    for (int w = 0; w < wave; ++w) base += wave_totals[w];
+    for (int i = begin; i < end; ++i) {
+        base += counts[i];
+        counts[i] = base;
+    }
+    if (tid == 0) row_ptr[0] = 0;
+}
+
+__global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__restrict__ dense, int rows,
+                                                           int cols, const int *__restrict__ row_ptr,
+                                                           uint16_t *__restrict__ values,
+                                                           unsigned char *__restrict__ deltas)
+{
+    __shared__ uint16_t stage_values[kRowsPerBlock][kTile];
+    __shared__ unsigned char stage_nibbles[kRowsPerBlock][kTile];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = uniform(threadIdx.x >> 6);
+    const int row = blockIdx.x * kRowsPerBlock + wave;
+    const bool live = row < rows;
+    const int e0 = live ? row_ptr[row] : 0;
+    const int e1 = live ? row_ptr[row + 1] : 0;
+    const uint16_t *src = dense + (size_t)(live ? row : 0) * (size_t)cols;
+    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+    uint16_t *sv = stage_values[wave];
+    unsigned char *sn = stage_nibbles[wave];
+    u32 *words = reinterpret_cast<u32 *>(deltas);
+
+    int carry = -1;
+    int pos = e0;  // next entry index to write
+    for (int c0 = 0; c0 < cols; c0 += kTile) {
+        int n_write = 0;
+        if (pos < e1) {  // wave-uniform
+            const int col = c0 + lane * kChunk;
+            const u32x4 v = load8(src, col, cols, vector_ok && col < cols);
+            const u32 nz = nonzero_bits(v);
+            const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
+            int pass_last;
+            int p = previous_nonzero(own_last, carry, lane, pass_last);
+            carry = pass_last > carry ? pass_last : carry;
+            // which of my 8 columns store an entry, and with which nibble
+            u32 entry_bits = 0;
+            u32 nibbles = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int x = col + i;
+                const int dist = x - p;
+                const bool is_nz = (nz >> i) & 1u;
+                const bool is_entry = x < cols && (is_nz || (dist & 15) == 0);
+                const u32 nib = is_nz ? (u32)(dist - 1) & 15u : 15u;
+                entry_bits |= (is_entry ? 1u : 0u) << i;
+                nibbles |= nib << (4 * i);
+                p = is_nz ? x : p;
+            }
+            const int mine = __builtin_popcount(entry_bits);
+            const int incl = wave_scan_inclusive(mine);
+            const int produced = __builtin_amdgcn_readlane(incl, kWave - 1);
+            int slot = incl - mine;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (entry_bits & (1u << i)) {
+                    u32 h = half_at(v, i);
+                    h = (h & 0x7fffu) > 0x7c00u ? 0x7fffu : h;
+                    sv[slot] = (uint16_t)h;
+                    sn[slot] = (unsigned char)((nibbles >> (4 * i)) & 15u);
+                    ++slot;
+                }
+            }
+            // entries past e1 are padding entries behind the row's last non-zero: not stored
+            n_write = produced < e1 - pos ? produced : e1 - pos;
+        }
+        __syncthreads();  // staged entries visible to the whole wave
+        if (n_write > 0) {
+            for (int k = lane; k < n_write; k += kWave) values[pos + k] = sv[k];
+            // nibble pairs that live wholly inside [pos, pos + n_write) are plain byte stores;
+            // a lone nibble at either end shares its byte with a neighbour and is OR-ed in
+            const int first_even = pos + (pos & 1);
+            const int last_even = (pos + n_write) & ~1;
+            for (int e = first_even + 2 * lane; e < last_even; e += 2 * kWave)
+                deltas[e >> 1] = (unsigned char)(sn[e - pos] | (sn[e + 1 - pos] << 4));
+            if (lane == 0 && (pos & 1)) {
+                const int byte = pos >> 1;
+                atomicOr(&words[byte >> 2], ((u32)sn[0] << 4) << (8 * (byte & 3)));
+            }
+            if (lane == 1 && ((pos + n_write) & 1)) {
+                const int e = pos + n_write - 1;
+                const int byte = e >> 1;
+                atomicOr(&words[byte >> 2], (u32)sn[e - pos] << (8 * (byte & 3)));
+            }
+            pos += n_write;
+        }
+        __syncthreads();  // staging buffers are reused by the next pass
+    }
+}
+
+// One wave per row, one entry per lane per pass.
+__global__ void __launch_bounds__(kBlock) decode_rows_kernel(const uint16_t *__restrict__ values,
+                                                             const unsigned char *__restrict__ deltas,
+                                                             const int *__restrict__ row_ptr, int rows, int cols,
+                                                             uint16_t *__restrict__ dense)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + uniform(threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int e0 = row_ptr[row];
+    const int e1 = row_ptr[row + 1];
+    uint16_t *dst = dense + (size_t)row * (size_t)cols;
+    int column = -1;  // column of the last entry decoded so far
+    for (int j0 = e0; j0 < e1; j0 += kWave) {
+        const int j = j0 + lane;
+        int step = 0;
+        uint16_t val = 0;
+        if (j < e1) {
+            step = ((deltas[j >> 1] >> (4 * (j & 1))) & 15) + 1;
+            val = values[j];
+        }
+        const int incl = wave_scan_inclusive(step);
+        const int c = column + incl;
+        if (j < e1 && c < cols) dst[c] = val;
+        column += __builtin_amdgcn_readlane(incl, kWave - 1);
+    }
+}
+
+}  // namespace
+}  // namespace macko
+
+extern "C" int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                        void *stream)
+{
+    using namespace macko;
+    if (rows < 0 || cols < 0 || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
+    if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
+    if (rows > 0 && cols > 0 && dense == nullptr) return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(row_ptr) & 3))
+        return MACKO_E_INVALID_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    if (rows > 0) {
+        hipLaunchKernelGGL(count_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0,
+                           s, (const uint16_t *)dense, rows, cols, row_ptr + 1);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, s, row_ptr, rows);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,
+                                       void *values, void *deltas, int64_t padded_entries, void *stream)
+{
+    using namespace macko;
+    if (rows < 0 || cols < 0 || padded_entries < 0 || padded_entries % kChunk != 0)
+        return MACKO_E_INVALID_ARGUMENT;
+    if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
+    if (padded_entries == 0) return 0;
+    if (dense == nullptr || row_ptr == nullptr || values == nullptr || deltas == nullptr)
+        return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(values) & 1) ||
+        (reinterpret_cast<uintptr_t>(deltas) & 3))
+        return MACKO_E_INVALID_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    hipError_t e = hipMemsetAsync(values, 0, (size_t)padded_entries * 2, s);
+    if (e != hipSuccess) return (int)e;
+    e = hipMemsetAsync(deltas, 0, (size_t)padded_entries / 2, s);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(fill_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
+                       (const uint16_t *)dense, rows, cols, row_ptr, (uint16_t *)values, (unsigned char *)deltas);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr, int32_t rows,
+                                    int32_t cols, void *dense, void *stream)
+{
+    using namespace macko;
+    if (rows < 0 || cols < 0) return MACKO_E_INVALID_ARGUMENT;
+    if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
+    if (rows == 0 || cols == 0) return 0;
+    if (dense == nullptr || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    hipError_t e = hipMemsetAsync(dense, 0, (size_t)rows * (size_t)cols * 2, s);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(decode_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
+                       (const uint16_t *)values, (const unsigned char *)deltas, row_ptr, rows, cols,
+                       (uint16_t *)dense);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,161 @@
+// PyTorch-ROCm binding of the MACKO path: registers the `macko_spmv` operator library and
+// forwards to the C ABI of libmacko_hip.so on torch's current HIP stream.
+//
+// Mirrors the upstream torch boundary:
+//   macko_spmv::multiply  <- TORCH_LIBRARY block in src/macko_spmv/__init__.py:56-63 and
+//                            macko_spmv_launcher, src/macko_spmv/cuda/kernels_torch_launchers.cuh:3-48
+//   macko_spmv::compress  <- cpu_compress, src/macko_spmv/cuda/cpu_compressor_torch_launcher.cuh:6-39
+// HIP tensors dispatch on the CUDA key in PyTorch-ROCm.  There is deliberately no CPU kernel
+// for multiply: without a GPU the operator raises.
+
+#include <ATen/ATen.h>
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <tuple>
+
+#include "macko_hip.h"
+
+namespace {
+
+void check_rc(int rc, const char *what)
+{
+    TORCH_CHECK(rc == 0, "macko_spmv: ", what, " failed: ", macko_hip_error_string(rc), " (code ", rc, ")");
+}
+
+at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                        int64_t M_rows, int64_t M_cols, const at::Tensor &V)
+{
+    TORCH_CHECK(M_values.dtype() == at::kHalf, "M must be torch.half");
+    TORCH_CHECK(V.dtype() == at::kHalf, "V must be torch.half");
+    TORCH_CHECK(M_deltas.dtype() == at::kByte, "M_deltas must be torch.uint8");
+    TORCH_CHECK(M_row_indices.dtype() == at::kInt, "M_row_indices must be torch.int32");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda(),
+                "all tensors must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
+                    V.is_contiguous(),
+                "all tensors must be contiguous");
+    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
+    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
+    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+    TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
+
+    const c10::hip::HIPGuard guard(M_values.device());
+    at::Tensor C = at::empty({M_rows}, M_values.options());
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    const int rc = macko_spmv_f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                  V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols,
+                                  M_values.numel(), (void *)stream);
+    check_rc(rc, "multiply");
+    return C;
+}
+
+// C = alpha * (M @ V) + beta * C, in place on C.
+void multiply_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                        int64_t M_rows, int64_t M_cols, const at::Tensor &V, at::Tensor C, double alpha,
+                        double beta)
+{
+    TORCH_CHECK(M_values.dtype() == at::kHalf && V.dtype() == at::kHalf && C.dtype() == at::kHalf,
+                "M, V and C must be torch.half");
+    TORCH_CHECK(M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt, "bad index dtypes");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda() && C.is_cuda(),
+                "all tensors must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
+                    V.is_contiguous() && C.is_contiguous(),
+                "all tensors must be contiguous");
+    TORCH_CHECK(C.numel() >= M_rows && M_row_indices.numel() >= M_rows + 1, "bad sizes");
+    TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
+    const c10::hip::HIPGuard guard(M_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    const int rc = macko_spmv_f16_axpby(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                        V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols,
+                                        M_values.numel(), (float)alpha, (float)beta, (void *)stream);
+    check_rc(rc, "multiply_axpby");
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_on_device(const at::Tensor &M)
+{
+    const c10::hip::HIPGuard guard(M.device());
+    const int64_t rows = M.size(0), cols = M.size(1);
+    TORCH_CHECK(rows * cols < (1ll << 31), "matrix too large: rows * cols must stay below 2^31");
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    at::Tensor row_ptr = at::empty({rows + 1}, M.options().dtype(at::kInt));
+    check_rc(macko_compress_f16_count(M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(),
+                                      (void *)stream),
+             "compress (count)");
+    const int64_t n = row_ptr[rows].item<int>();  // one 4-byte read-back; sizes the outputs
+    const int64_t padded = (n + 7) / 8 * 8;
+    at::Tensor values = at::empty({padded}, M.options());
+    at::Tensor deltas = at::empty({padded / 2}, M.options().dtype(at::kByte));
+    check_rc(macko_compress_f16_fill(M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(),
+                                     values.data_ptr(), deltas.data_ptr(), padded, (void *)stream),
+             "compress (fill)");
+    return std::make_tuple(values, deltas, row_ptr, rows, cols);
+}
+
+// HIP tensor in -> HIP tensors out.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_hip(const at::Tensor &M)
+{
+    TORCH_CHECK(M.dtype() == at::kHalf, "M must be torch.half");
+    TORCH_CHECK(M.dim() == 2, "M must be a matrix");
+    TORCH_CHECK(M.is_contiguous(), "M must be contiguous");
+    return compress_on_device(M);
+}
+
+// CPU tensor in -> CPU tensors out, like the upstream cpu_compress, but the work is done by the
+// HIP compressor: the matrix is staged to the current GPU and the three arrays are copied back.
+// Needs a GPU; there is no host implementation.
+std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_cpu(const at::Tensor &M)
+{
+    TORCH_CHECK(M.dtype() == at::kHalf, "M must be torch.half");
+    TORCH_CHECK(M.dim() == 2, "M must be a matrix");
+    TORCH_CHECK(M.is_contiguous(), "M must be contiguous");
+    int n_dev = 0;
+    TORCH_CHECK(hipGetDeviceCount(&n_dev) == hipSuccess && n_dev > 0,
+                "macko_spmv: compress needs an AMD GPU (the compressor is a HIP kernel; there is no CPU path)");
+    auto out = compress_on_device(M.to(at::Device(at::kCUDA, c10::hip::current_device())));
+    return std::make_tuple(std::get<0>(out).cpu(), std::get<1>(out).cpu(), std::get<2>(out).cpu(),
+                           std::get<3>(out), std::get<4>(out));
+}
+
+at::Tensor decompress_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                          int64_t M_rows, int64_t M_cols)
+{
+    TORCH_CHECK(M_values.dtype() == at::kHalf && M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt,
+                "bad dtypes");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
+                "all tensors must be contiguous");
+    const c10::hip::HIPGuard guard(M_values.device());
+    at::Tensor dense = at::empty({M_rows, M_cols}, M_values.options());
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    check_rc(macko_decompress_f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                  (int32_t)M_rows, (int32_t)M_cols, dense.data_ptr(), (void *)stream),
+             "decompress");
+    return dense;
+}
+
+}  // namespace
+
+TORCH_LIBRARY(macko_spmv, m)
+{
+    // same schema string as the upstream package
+    m.def("multiply(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, Tensor V) -> Tensor");
+    m.def("multiply_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
+    m.def("compress(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
+    m.def("decompress(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols) -> Tensor");
+}
+
+TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
+{
+    m.impl("multiply", &multiply_hip);
+    m.impl("multiply_axpby", &multiply_axpby_hip);
+    m.impl("compress", &compress_hip);
+    m.impl("decompress", &decompress_hip);
+}
+
+TORCH_LIBRARY_IMPL(macko_spmv, CPU, m)
+{
+    m.impl("compress", &compress_cpu);
+}

@@ -1,0 +1,126 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports what its header
+declares, argument validation returns before anything touches a device, and the Python/torch
+boundary behaves like the upstream package's (exception types, fake implementation, schema)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import macko_spmv
+import macko_spmv_amd
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "macko_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(macko_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = _declared_symbols()
+    assert {"macko_spmv_f16", "macko_spmv_f16_axpby", "macko_compress_f16_count", "macko_compress_f16_fill",
+            "macko_decompress_f16", "macko_hip_error_string", "macko_hip_abi_version"} <= set(names)
+    lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in include/macko_hip.h but not exported"
+
+
+def test_abi_version_and_error_strings():
+    lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
+    assert lib.macko_hip_abi_version() == 1
+    lib.macko_hip_error_string.restype = ctypes.c_char_p
+    assert lib.macko_hip_error_string(0) == b"success"
+    assert b"invalid argument" in lib.macko_hip_error_string(-1)
+    assert b"no usable HIP device" in lib.macko_hip_error_string(-2)
+    assert lib.macko_hip_error_string(-99)
+
+
+def test_argument_validation_needs_no_device():
+    lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
+    vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+    lib.macko_spmv_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i64, vp]
+    lib.macko_compress_f16_count.argtypes = [vp, i32, i32, vp, vp]
+    lib.macko_compress_f16_fill.argtypes = [vp, i32, i32, vp, vp, vp, i64, vp]
+    assert lib.macko_spmv_f16(None, None, None, None, None, -1, 4, 0, None) == -1      # negative rows
+    assert lib.macko_spmv_f16(None, None, None, None, None, 4, 4, 8, None) == -1       # null pointers
+    assert lib.macko_spmv_f16(16, 16, 16, 16, 16, 4, 4, 12, None) == -1                # P not a multiple of 8
+    assert lib.macko_spmv_f16(8, 16, 16, 16, 16, 4, 4, 8, None) == -1                  # values not 16-byte aligned
+    assert lib.macko_spmv_f16(None, None, None, None, None, 0, 0, 0, None) == 0        # nothing to do
+    assert lib.macko_compress_f16_count(None, 4, 4, None, None) == -1
+    assert lib.macko_compress_f16_count(16, 65536, 65536, 16, None) == -1              # rows*cols >= 2^31
+    assert lib.macko_compress_f16_fill(None, 4, 4, None, None, None, 0, None) == 0     # empty output
+    assert lib.macko_compress_f16_fill(None, 4, 4, None, None, None, 8, None) == -1
+
+
+def test_alias_package_exposes_the_upstream_surface():
+    for name in ("compress", "multiply", "move_to_device"):
+        assert getattr(macko_spmv, name) is getattr(macko_spmv_amd, name)
+
+
+def test_operator_schema_matches_upstream():
+    schema = str(torch.ops.macko_spmv.multiply.default._schema)
+    assert schema == ("macko_spmv::multiply(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, "
+                      "int M_rows, int M_cols, Tensor V) -> Tensor")
+
+
+def test_fake_implementation_shapes():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        values = torch.empty(16, dtype=torch.float16, device="cuda")
+        deltas = torch.empty(8, dtype=torch.uint8, device="cuda")
+        row_ptr = torch.empty(6, dtype=torch.int32, device="cuda")
+        x = torch.empty(32, dtype=torch.float16, device="cuda")
+        y = torch.ops.macko_spmv.multiply(values, deltas, row_ptr, 5, 32, x)
+        assert y.shape == (5,) and y.dtype == torch.float16 and y.device.type == "cuda"
+
+
+def test_multiply_rejects_cpu_tensors_with_assertion():
+    compressed = (torch.zeros(8, dtype=torch.float16), torch.zeros(4, dtype=torch.uint8),
+                  torch.zeros(2, dtype=torch.int32), 1, 8)
+    with pytest.raises(AssertionError):
+        macko_spmv.multiply(compressed, torch.zeros(8, dtype=torch.float16))
+
+
+def test_multiply_has_no_cpu_kernel():
+    # the operator must fail loudly rather than fall back to a host implementation
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.macko_spmv.multiply(torch.zeros(8, dtype=torch.float16), torch.zeros(4, dtype=torch.uint8),
+                                      torch.zeros(2, dtype=torch.int32), 1, 8, torch.zeros(8, dtype=torch.float16))
+
+
+def test_compress_argument_errors():
+    with pytest.raises(AssertionError):  # non-contiguous input (upstream: assert M.is_contiguous())
+        macko_spmv.compress(torch.zeros(8, 8, dtype=torch.float16).t()[:, ::2])
+    with pytest.raises(NotImplementedError):  # neither cpu nor cuda
+        macko_spmv.compress(torch.zeros(4, 4, dtype=torch.float16, device="meta"))
+    with pytest.raises(RuntimeError, match="torch.half"):  # dtype check of the launcher
+        macko_spmv.compress(torch.zeros(4, 4, dtype=torch.float32))
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="only meaningful without a GPU")
+def test_compress_without_gpu_raises():
+    with pytest.raises(RuntimeError, match="needs an AMD GPU"):
+        macko_spmv.compress(torch.zeros(4, 8, dtype=torch.float16))
+
+
+def test_move_to_device_keeps_ints():
+    compressed = (torch.zeros(8, dtype=torch.float16), torch.zeros(4, dtype=torch.uint8),
+                  torch.zeros(2, dtype=torch.int32), 1, 8)
+    moved = macko_spmv.move_to_device(compressed, "cpu")
+    assert len(moved) == 5 and moved[3] == 1 and moved[4] == 8
+    assert all(t.device.type == "cpu" for t in moved[:3])
+
+
+def test_product_package_does_not_touch_the_oracle():
+    pkg = os.path.join(ROOT, "macko_spmv_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith((".py", ".hip", ".cpp", ".h")):
+                text = open(os.path.join(dirpath, name)).read()
+                assert "oracle" not in text, f"{name} mentions the oracle"
