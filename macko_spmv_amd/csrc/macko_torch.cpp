@@ -5,12 +5,13 @@
 //   macko_spmv::multiply  <- TORCH_LIBRARY block in src/macko_spmv/__init__.py:56-63 and
 //                            macko_spmv_launcher, src/macko_spmv/cuda/kernels_torch_launchers.cuh:3-48
 //   macko_spmv::compress  <- cpu_compress, src/macko_spmv/cuda/cpu_compressor_torch_launcher.cuh:6-39
-// HIP tensors dispatch on the CUDA key in PyTorch-ROCm.  There is deliberately no CPU kernel
+// HIP tensors carry the "cuda" device type and dispatch on the CUDA key in PyTorch-ROCm, hence
+// the *MasqueradingAsCUDA guard and stream accessors.  There is deliberately no CPU kernel
 // for multiply: without a GPU the operator raises.
 
 #include <ATen/ATen.h>
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
 #include <tuple>
@@ -41,9 +42,9 @@ at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
     TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
     TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
 
-    const c10::hip::HIPGuard guard(M_values.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
     at::Tensor C = at::empty({M_rows}, M_values.options());
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const int rc = macko_spmv_f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
                                   V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols,
                                   M_values.numel(), (void *)stream);
@@ -66,8 +67,8 @@ void multiply_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
                 "all tensors must be contiguous");
     TORCH_CHECK(C.numel() >= M_rows && M_row_indices.numel() >= M_rows + 1, "bad sizes");
     TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
-    const c10::hip::HIPGuard guard(M_values.device());
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const int rc = macko_spmv_f16_axpby(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
                                         V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols,
                                         M_values.numel(), (float)alpha, (float)beta, (void *)stream);
@@ -76,10 +77,10 @@ void multiply_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
 
 std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_on_device(const at::Tensor &M)
 {
-    const c10::hip::HIPGuard guard(M.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M.device());
     const int64_t rows = M.size(0), cols = M.size(1);
     TORCH_CHECK(rows * cols < (1ll << 31), "matrix too large: rows * cols must stay below 2^31");
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     at::Tensor row_ptr = at::empty({rows + 1}, M.options().dtype(at::kInt));
     check_rc(macko_compress_f16_count(M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(),
                                       (void *)stream),
@@ -126,9 +127,9 @@ at::Tensor decompress_hip(const at::Tensor &M_values, const at::Tensor &M_deltas
                 "bad dtypes");
     TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
                 "all tensors must be contiguous");
-    const c10::hip::HIPGuard guard(M_values.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
     at::Tensor dense = at::empty({M_rows, M_cols}, M_values.options());
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_rc(macko_decompress_f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
                                   (int32_t)M_rows, (int32_t)M_cols, dense.data_ptr(), (void *)stream),
              "decompress");

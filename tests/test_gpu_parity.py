@@ -156,12 +156,21 @@ def test_multiply_upstream_random_sweep(density, seed):
     M = M_cpu.cuda()
     V = torch.rand((8192,), device="cuda", dtype=torch.float16)
     compressed = macko_spmv.compress(M)
-    if density == 0:
-        assert compressed[0].numel() == 0 and compressed[1].numel() == 0
     got = macko_spmv.multiply(compressed, V)
     assert torch.allclose(M @ V, got, rtol=1e-3, atol=1e-3), f"Fail at {seed} {density}"
     want = (M_cpu.double() @ V.cpu().double()).numpy()
     helpers.assert_close_fp16(got.cpu().numpy(), want)
+
+
+def test_all_zero_matrix_gives_empty_arrays_and_zero_product():
+    M = torch.zeros((300, 777), dtype=torch.float16, device="cuda")
+    M[5, 5] = -0.0
+    compressed = macko_spmv.compress(M)
+    assert compressed[0].numel() == 0 and compressed[1].numel() == 0
+    assert torch.equal(compressed[2].cpu(), torch.zeros(301, dtype=torch.int32))
+    V = torch.full((777,), float("inf"), dtype=torch.float16, device="cuda")
+    y = macko_spmv.multiply(compressed, V)
+    assert y.shape == (300,) and not y.any()
 
 
 def test_multiply_small_and_ragged_shapes():
