@@ -1,15 +1,22 @@
 // MACKO fp16 sparse matrix-vector product for gfx950 (wave64).
 //
-// Work split.  The launch has W = gridDim.x * (BLOCK/64) waves.  Wave w owns the rows whose
-// first entry index lies in [w*P/W, (w+1)*P/W): contiguous whole rows, balanced by stored
-// entries, found by a 64-wide search of row_ptr.  No two waves share a row, so there is no
-// cross-wave reduction and no scratch memory.
+// Data movement.  The value and delta arrays are cut into fixed tiles of 512 entries (one
+// 128-bit value load and one 32-bit delta load per lane).  The launch has W waves; wave w
+// streams the tiles [w*NT/W, (w+1)*NT/W) and a little beyond, keeping D tiles in flight in a
+// register ring.  Because tile positions do not depend on row_ptr, the first D loads are issued
+// at the top of the kernel, together with the row_ptr probe and the copy of x into LDS: one
+// memory latency, not a chain of them, sits in front of the first multiply-add.
 //
-// Per row a wave walks the row's 8-entry chunks 64 at a time (one chunk per lane: one 128-bit
-// value load and one 32-bit delta load), D such passes in flight.  Columns come from a DPP
-// prefix sum over per-lane nibble sums plus v_dot8_u32_u4 for the running sum inside a lane; the
-// dense vector is gathered from LDS, where the workgroup staged it once.  fp32 accumulation,
-// one DPP reduction per row, fp16 store.
+// Row ownership.  Wave w owns the rows whose first entry index lies inside its nominal tile
+// range (contiguous whole rows, balanced by stored entries, found with a 64-wide search of
+// row_ptr).  It walks from the tile holding its first owned entry to the tile holding its last,
+// which overlaps the neighbours' nominal ranges by at most one row.  No row is shared between
+// waves, so there is no cross-wave reduction, no atomics and no scratch memory.
+//
+// Per tile, the entries of one row form a segment [first lane/entry, last lane/entry]; each
+// segment takes one pass: mask, DPP prefix sum of per-lane nibble sums, v_dot8_u32_u4 for the
+// running sum inside a lane, gather of x from LDS, fp32 FMA.  A row ends with one DPP
+// reduction and an fp16 store.
 //
 // Behaviour restated from src/macko_spmv/cuda/kernels.cuh:34-124 of the upstream package.
 
@@ -20,6 +27,8 @@ namespace {
 
 constexpr int kLdsFront = 16;   // zero bytes in front of x in LDS (masked head entries read here)
 constexpr int kLdsBack = 64;    // zero bytes behind x (masked tail entries read here)
+constexpr int kTileShift = 9;   // log2(kTile)
+constexpr int kXRegs = 2;       // 16-byte pieces of x a thread carries in registers while staging
 
 struct SpmvArgs {
     const u32 *values;      // fp16 pairs
@@ -32,7 +41,14 @@ struct SpmvArgs {
     long long padded;       // P
     float alpha;
     float beta;
+    // split of tiles and rows over the launch's waves, precomputed on the host so the kernel
+    // does no 64-bit division: wave w starts at w*q + min(w, rem)
+    u32 n_tiles, tiles_q, tiles_rem;
+    u32 rows_q, rows_rem;
 };
+
+// First item of wave w when n items are dealt to the waves as evenly as possible.
+__device__ __forceinline__ u32 even_split(u32 w, u32 q, u32 rem) { return w * q + (w < rem ? w : rem); }
 
 __device__ __forceinline__ float half_bits_to_float(uint16_t h)
 {
@@ -44,57 +60,66 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float f)
     return __builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
-// Smallest r in [0, rows] with row_ptr[r] >= target (rows if there is none), for two targets
-// at once.  All 64 lanes probe together; `guess` centres the first probe window, which hits
-// when rows carry similar entry counts.  Every value here is wave-uniform.
+// Where the first probe of the row search looks: 64 consecutive row_ptr values starting a few
+// rows before `guess`.
+__device__ __forceinline__ int probe_base(int guess, int rows)
+{
+    int w0 = guess - 8;
+    const int wmax = rows - 63;
+    w0 = w0 > wmax ? wmax : w0;
+    return w0 < 0 ? 0 : w0;
+}
+
+// Lane i of the returned value holds row_ptr[base + i] (row_ptr[rows] beyond the end).
+__device__ __forceinline__ int load_row_window(const int *__restrict__ row_ptr, int rows, int base, int lane)
+{
+    const int idx = base + lane;
+    return row_ptr[idx <= rows ? idx : rows];
+}
+
+// Smallest r in [0, rows] with row_ptr[r] >= target (rows if there is none), for two targets at
+// once.  All 64 lanes probe together.  window[k] is an already loaded probe (see
+// load_row_window) at base[k]; it resolves the search when rows carry similar entry counts,
+// otherwise 64-ary rounds follow.  Every value here is wave-uniform.
 __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_ptr, int rows, int lane,
-                                                  const int target[2], const int guess[2], int out[2])
+                                                  const int target[2], const int window[2], const int base[2],
+                                                  int out[2])
 {
     int lo[2], hi[2];
-    int probe[2], win[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-        int w0 = guess[k] - 32;
-        int wmax = rows - 63;
-        w0 = w0 > wmax ? wmax : w0;
-        w0 = w0 < 0 ? 0 : w0;
-        win[k] = w0;
-        int idx = w0 + lane;
-        probe[k] = idx <= rows ? row_ptr[idx] : 0x7fffffff;
-    }
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        unsigned long long m = __ballot(probe[k] >= target[k]);
+        const bool beyond = base[k] + lane > rows;
+        const unsigned long long m = __ballot(beyond || window[k] >= target[k]);
         if (m == 0) {  // everything probed is below the target
-            lo[k] = win[k] + 64 > rows ? rows : win[k] + 64;
+            lo[k] = base[k] + 64 > rows ? rows : base[k] + 64;
             hi[k] = rows;
         } else {
-            int f = __builtin_ctzll(m);
+            const int f = __builtin_ctzll(m);
             if (f == 0) {  // the answer is at or before the window start
                 lo[k] = 0;
-                hi[k] = win[k];
+                hi[k] = base[k];
             } else {
-                lo[k] = hi[k] = win[k] + f > rows ? rows : win[k] + f;
+                lo[k] = hi[k] = base[k] + f > rows ? rows : base[k] + f;
             }
         }
     }
     while (lo[0] < hi[0] || lo[1] < hi[1]) {
-        int step[2];
+        int step[2], probe[2];
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             step[k] = (hi[k] - lo[k] + 63) >> 6;
-            int idx = lo[k] + lane * step[k];
+            const int idx = lo[k] + lane * step[k];
             probe[k] = (lo[k] < hi[k] && idx < hi[k]) ? row_ptr[idx] : 0x7fffffff;
         }
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             if (lo[k] < hi[k]) {
-                unsigned long long m = __ballot(probe[k] >= target[k]);
+                const unsigned long long m = __ballot(probe[k] >= target[k]);
                 if (m == 0) {
                     lo[k] = lo[k] + 63 * step[k] + 1;
                 } else {
-                    int f = __builtin_ctzll(m);
-                    int at = lo[k] + f * step[k];
+                    const int f = __builtin_ctzll(m);
+                    const int at = lo[k] + f * step[k];
                     if (f > 0) lo[k] = lo[k] + (f - 1) * step[k] + 1;
                     if (at < hi[k]) hi[k] = at;
                 }
@@ -106,29 +131,12 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
     out[1] = lo[1];
 }
 
-// Copy x[0..cols) into LDS behind kLdsFront zero bytes and put kLdsBack zero bytes after it.
-template <int BLOCK>
-__device__ __forceinline__ void stage_x(unsigned char *lds, const uint16_t *__restrict__ x, int cols, int tid)
+// 128-bit mask helpers: keep halves [from, 8) / [0, upto) of a 4-dword vector and the matching
+// nibbles.  `from` / `upto` are wave-uniform, so the masks are built on the scalar unit.
+__device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)  // 1 <= from <= 7
 {
-    uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
-    if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-    if (tid < kLdsBack / 2) dst[cols + tid] = 0;
-    if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-        const int nvec = cols >> 3;
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(x);
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
-        for (int i = tid; i < nvec; i += BLOCK) d4[i] = src[i];
-        for (int i = (nvec << 3) + tid; i < cols; i += BLOCK) dst[i] = x[i];
-    } else {
-        for (int i = tid; i < cols; i += BLOCK) dst[i] = x[i];
-    }
-}
-
-// 128-bit mask helpers: keep halves [from, 8) / [0, upto) of a 4-dword vector.
-__device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)
-{
-    unsigned long long lo = from < 4 ? (~0ull << (16 * from)) : 0ull;
-    unsigned long long hi = from < 4 ? ~0ull : (~0ull << (16 * (from - 4)));
+    const unsigned long long lo = from < 4 ? (~0ull << (16 * from)) : 0ull;
+    const unsigned long long hi = from < 4 ? ~0ull : (~0ull << (16 * (from - 4)));
     v.x &= (u32)lo;
     v.y &= (u32)(lo >> 32);
     v.z &= (u32)hi;
@@ -138,8 +146,8 @@ __device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)
 
 __device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= upto <= 7
 {
-    unsigned long long lo = upto < 4 ? ((1ull << (16 * upto)) - 1) : ~0ull;
-    unsigned long long hi = upto <= 4 ? 0ull : ((1ull << (16 * (upto - 4))) - 1);
+    const unsigned long long lo = upto < 4 ? ((1ull << (16 * upto)) - 1) : ~0ull;
+    const unsigned long long hi = upto <= 4 ? 0ull : ((1ull << (16 * (upto - 4))) - 1);
     v.x &= (u32)lo;
     v.y &= (u32)(lo >> 32);
     v.z &= (u32)hi;
@@ -148,36 +156,49 @@ __device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= u
 }
 
 template <int BLOCK, int D, bool X_LDS, bool AXPBY>
-__global__ void __launch_bounds__(BLOCK) spmv_rows_kernel(const SpmvArgs a)
+__global__ void __launch_bounds__(BLOCK) spmv_stream_kernel(const SpmvArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int WAVES = BLOCK / kWave;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = uniform(tid >> 6);
-    const int n_waves = gridDim.x * WAVES;
-    const int gw = blockIdx.x * WAVES + wave;
+    const u32 n_waves = gridDim.x * WAVES;
+    const u32 gw = blockIdx.x * WAVES + wave;
 
-    // ---- which rows are mine -------------------------------------------------------------
-    int range[2];
+    const u32 nt_lo = even_split(gw, a.tiles_q, a.tiles_rem);
+    const u32 nt_hi = even_split(gw + 1, a.tiles_q, a.tiles_rem);
+
+    // Loads are issued in the order probe, x, tiles; they complete in that order, so each
+    // consumer below waits only for what was issued before its own data.
+
+    // ---- 1. row_ptr probe ---------------------------------------------------------------------
+    int target[2], base[2], window[2];
     {
-        int target[2], guess[2];
-        target[0] = (int)(((long long)gw * a.padded) / n_waves);
-        target[1] = (int)(((long long)(gw + 1) * a.padded) / n_waves);
-        guess[0] = (int)(((long long)gw * a.rows) / n_waves);
-        guess[1] = (int)(((long long)(gw + 1) * a.rows) / n_waves);
-        wave_lower_bound2(a.row_ptr, a.rows, lane, target, guess, range);
-        if (gw == 0) range[0] = 0;
-        if (gw == n_waves - 1) range[1] = a.rows;
+        const unsigned long long t0 = (unsigned long long)nt_lo << kTileShift;
+        const unsigned long long t1 = (unsigned long long)nt_hi << kTileShift;
+        target[0] = t0 > 0x7fffffffull ? 0x7fffffff : (int)t0;
+        target[1] = t1 > 0x7fffffffull ? 0x7fffffff : (int)t1;
+        base[0] = probe_base((int)even_split(gw, a.rows_q, a.rows_rem), a.rows);
+        base[1] = probe_base((int)even_split(gw + 1, a.rows_q, a.rows_rem), a.rows);
+        window[0] = load_row_window(a.row_ptr, a.rows, base[0], lane);
+        window[1] = load_row_window(a.row_ptr, a.rows, base[1], lane);
     }
-    const int row_first = uniform(range[0]);
-    const int row_last = uniform(range[1]);
 
+    // ---- 2. x: the first pieces travel through registers ---------------------------------------
+    const bool x_vec = (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+    const int x_nvec = x_vec ? a.cols >> 3 : 0;
+    u32x4 xr[kXRegs];
     if (X_LDS) {
-        stage_x<BLOCK>(lds, a.x, a.cols, tid);
-        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kXRegs; ++j) {
+            const int i = tid + j * BLOCK;
+            xr[j] = (u32x4){0, 0, 0, 0};
+            if (i < x_nvec) xr[j] = reinterpret_cast<const u32x4 *>(a.x)[i];
+        }
     }
 
+    // ---- 3. the first D tiles of my nominal range -----------------------------------------------
     const __amdgpu_buffer_rsrc_t rs_values =
         __builtin_amdgcn_make_buffer_rsrc((void *)a.values, 0, (int)(u32)(a.padded * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_deltas =
@@ -185,86 +206,164 @@ __global__ void __launch_bounds__(BLOCK) spmv_rows_kernel(const SpmvArgs a)
     const __amdgpu_buffer_rsrc_t rs_x =
         __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.cols * 2, 0x00020000);
     (void)rs_x;
+    u32x4 v[D];
+    u32 d[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+        const u32 tile = nt_lo + j;
+        v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_values, lane * 16, (int)(tile << (kTileShift + 1)), 0);
+        d[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_deltas, lane * 4, (int)(tile << (kTileShift - 1)), 0);
+    }
 
-    for (int r0 = row_first; r0 < row_last; r0 += kWave - 1) {
-        const int batch = uniform(row_last - r0 < kWave - 1 ? row_last - r0 : kWave - 1);
-        int idx = r0 + lane;
-        idx = idx > a.rows ? a.rows : idx;
-        const int rp = a.row_ptr[idx];  // lane i: start of row r0 + i
-        for (int i = 0; i < batch; ++i) {
-            const int e0 = __builtin_amdgcn_readlane(rp, i);
-            const int e1 = __builtin_amdgcn_readlane(rp, i + 1);
-            float acc0 = 0.f, acc1 = 0.f;
-            if (e1 > e0) {
-                const int cb = e0 >> 3;
-                const int ce = (e1 + 7) >> 3;
-                const int head = e0 & 7;
-                const int tail = e1 & 7;
-                int carry = 0;  // nibble sum of the row so far
-                for (int c0 = cb; c0 < ce; c0 += kWave * D) {
-                    u32x4 v[D];
-                    u32 d[D];
+    // ---- 4. which rows are mine -------------------------------------------------------------------
+    int range[2];
+    wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
+    if (gw == n_waves - 1) range[1] = a.rows;
+    if (nt_lo == nt_hi) range[1] = range[0];  // no nominal tiles: owns nothing
+    const int row_first = uniform(range[0]);
+    const int row_last = uniform(range[1]);
+
+    // ---- 5. x into LDS ------------------------------------------------------------------------------
+    if (X_LDS) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
+        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
+        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
 #pragma unroll
-                    for (int j = 0; j < D; ++j) {
-                        const int t0 = c0 + kWave * j;
-                        v[j] = (u32x4){0, 0, 0, 0};
-                        d[j] = 0;
-                        if (t0 + lane < ce) {
-                            v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_values, lane * 16, (int)((u32)t0 * 16u), 0);
-                            d[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_deltas, lane * 4, t0 * 4, 0);
+        for (int j = 0; j < kXRegs; ++j) {
+            const int i = tid + j * BLOCK;
+            if (i < x_nvec) d4[i] = xr[j];
+        }
+        for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
+        for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
+        __syncthreads();
+    }
+
+    if (row_first >= row_last) return;
+
+    // ---- 6. stream --------------------------------------------------------------------------------
+    // window of row_ptr values: lane i holds row_ptr[win_base + i]
+    int win_base = base[0];
+    int win = window[0];
+    if (row_first < win_base || row_first + 1 > win_base + 63) {
+        win_base = row_first;
+        win = load_row_window(a.row_ptr, a.rows, win_base, lane);
+    }
+    auto row_start = [&](int r) -> int {  // r in [win_base, win_base + 63]
+        return __builtin_amdgcn_readlane(win, r - win_base);
+    };
+    auto slide_window = [&](int r) {  // make rows r and r + 1 addressable
+        if (r + 1 > win_base + 63) {
+            win_base = r;
+            win = load_row_window(a.row_ptr, a.rows, win_base, lane);
+        }
+    };
+    auto store_row = [&](int r, float total) {
+        if (lane == 0) {
+            float out = total;
+            if (AXPBY) out = a.alpha * total + a.beta * half_bits_to_float(a.y[r]);
+            a.y[r] = float_to_half_bits(out);
+        }
+    };
+
+    // current row r = first non-empty owned row; empty ones are written on the way
+    int r = row_first;
+    int e0 = row_start(r);
+    int e1 = row_start(r + 1);
+    while (e1 == e0) {
+        store_row(r, 0.f);
+        ++r;
+        if (r >= row_last) return;
+        slide_window(r);
+        e0 = row_start(r);
+        e1 = row_start(r + 1);
+    }
+    // end of my last owned row
+    const int s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
+    const u32 first_tile = (u32)e0 >> kTileShift;
+    const u32 last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
+
+    float acc0 = 0.f, acc1 = 0.f;
+    int carry = 0;  // nibble sum of the current row so far
+
+    for (u32 tile0 = nt_lo; tile0 < last_tile; tile0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            const u32 tile = tile0 + j;
+            if (tile >= last_tile) continue;  // wave-uniform
+            const u32x4 vj = v[j];
+            const u32 dj = d[j];
+            if (tile + D < last_tile) {  // refill this ring slot
+                v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_values, lane * 16,
+                                                              (int)((tile + D) << (kTileShift + 1)), 0);
+                d[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_deltas, lane * 4,
+                                                             (int)((tile + D) << (kTileShift - 1)), 0);
+            }
+            if (tile < first_tile) continue;  // fetched on speculation, belongs to the previous wave
+            const int tb = (int)(tile << kTileShift);
+            const int lim = tb + kTile < s_end ? tb + kTile : s_end;
+            int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
+            while (pos < lim) {
+                const int seg_end = e1 < lim ? e1 : lim;
+                // ---- one pass over the segment [pos, seg_end) of row r ----
+                const int rel0 = pos - tb;
+                const int rel1 = seg_end - tb;
+                u32x4 vv = vj;
+                u32 dd = dj;
+                bool active = true;
+                if (rel0 != 0 || rel1 != kTile) {  // not the whole tile (wave-uniform test)
+                    const int l0 = rel0 >> 3, q0 = rel0 & 7;
+                    const int l1 = (rel1 - 1) >> 3, q1 = rel1 & 7;
+                    active = lane >= l0 && lane <= l1;
+                    if (!active) dd = 0;
+                    if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
+                    if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
+                }
+                const int s = (int)__builtin_amdgcn_udot8(dd, 0x11111111u, 0u, false);
+                const int incl = wave_scan_inclusive(s);
+                const int excl = incl - s + carry;
+                carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+                if (active) {
+                    // LDS byte address of x[col] for entry 0 of this chunk, before its own nibble;
+                    // tb + 8*lane - e0 >= -7 for an active lane, so this stays positive
+                    const u32 addr0 = (u32)(kLdsFront + 2 * (tb + 8 * lane - e0 + excl));
+                    const u32 m[8] = {0x2u,     0x22u,     0x222u,     0x2222u,
+                                      0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const u32 addr = __builtin_amdgcn_udot8(dd, m[k], addr0, false);
+                        uint16_t xb;
+                        if (X_LDS) {
+                            xb = *reinterpret_cast<const uint16_t *>(lds + addr + 2 * k);
+                        } else {
+                            int o = (int)addr + 2 * k - kLdsFront;
+                            const int omax = 2 * a.cols - 2;
+                            o = o < 0 ? 0 : (o > omax ? omax : o);
+                            xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
                         }
-                    }
-#pragma unroll
-                    for (int j = 0; j < D; ++j) {
-                        const int t0 = c0 + kWave * j;
-                        if (t0 < ce) {
-                            u32x4 vj = v[j];
-                            u32 dj = d[j];
-                            if (t0 == cb && head != 0) {
-                                if (lane == 0) mask_from(vj, dj, head);
-                            }
-                            if (tail != 0 && ce - 1 - t0 < kWave) {
-                                if (lane == ce - 1 - t0) mask_upto(vj, dj, tail);
-                            }
-                            const int s = (int)__builtin_amdgcn_udot8(dj, 0x11111111u, 0u, false);
-                            const int incl = wave_scan_inclusive(s);
-                            const int excl = incl - s + carry;
-                            carry += __builtin_amdgcn_readlane(incl, kWave - 1);
-                            if (t0 + lane < ce) {
-                                // LDS byte address of x[col] for entry 0 of this chunk, before its own
-                                // nibble is added; 8c - e0 >= -7, so this stays positive
-                                const u32 base = (u32)(kLdsFront + 2 * (8 * (t0 + lane) - e0 + excl));
-                                const u32 m[8] = {0x2u,      0x22u,      0x222u,      0x2222u,
-                                                  0x22222u,  0x222222u,  0x2222222u,  0x22222222u};
-#pragma unroll
-                                for (int k = 0; k < 8; ++k) {
-                                    const u32 addr = __builtin_amdgcn_udot8(dj, m[k], base, false);
-                                    uint16_t xb;
-                                    if (X_LDS) {
-                                        xb = *reinterpret_cast<const uint16_t *>(lds + addr + 2 * k);
-                                    } else {
-                                        int o = (int)addr + 2 * k - kLdsFront;
-                                        const int omax = 2 * a.cols - 2;
-                                        o = o < 0 ? 0 : (o > omax ? omax : o);
-                                        xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
-                                    }
-                                    const u32 w = vj[k >> 1];
-                                    const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
-                                    if (k & 1)
-                                        acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
-                                    else
-                                        acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
-                                }
-                            }
-                        }
+                        const u32 w = vv[k >> 1];
+                        const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+                        if (k & 1)
+                            acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
+                        else
+                            acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
                     }
                 }
-            }
-            const float total = wave_sum(acc0 + acc1);
-            if (lane == 0) {
-                float out = total;
-                if (AXPBY) out = a.alpha * total + a.beta * half_bits_to_float(a.y[r0 + i]);
-                a.y[r0 + i] = float_to_half_bits(out);
+                // ---- row finished? ----
+                if (seg_end == e1) {
+                    store_row(r, wave_sum(acc0 + acc1));
+                    acc0 = acc1 = 0.f;
+                    carry = 0;
+                    do {  // next non-empty owned row; empty ones get their zero on the way
+                        ++r;
+                        if (r >= row_last) break;  // then seg_end == s_end == lim and both loops end
+                        slide_window(r);
+                        e0 = row_start(r);
+                        e1 = row_start(r + 1);
+                        if (e1 == e0) store_row(r, 0.f);
+                    } while (e1 == e0);
+                }
+                pos = seg_end;
             }
         }
     }
@@ -274,14 +373,20 @@ __global__ void __launch_bounds__(BLOCK) spmv_rows_kernel(const SpmvArgs a)
 template <bool AXPBY>
 __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
 {
-    int r = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
 template <int BLOCK, int D, bool X_LDS, bool AXPBY>
-int launch_rows(const SpmvArgs &a, int grid, size_t lds_bytes, hipStream_t stream)
+int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = spmv_rows_kernel<BLOCK, D, X_LDS, AXPBY>;
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY>;
+    const u32 n_waves = (u32)grid * (BLOCK / kWave);
+    a.n_tiles = (u32)((a.padded + kTile - 1) >> kTileShift);
+    a.tiles_q = a.n_tiles / n_waves;
+    a.tiles_rem = a.n_tiles % n_waves;
+    a.rows_q = (u32)a.rows / n_waves;
+    a.rows_rem = (u32)a.rows % n_waves;
     if (lds_bytes > 64 * 1024) {
         // one-time opt-in to more than 64 KiB of dynamic LDS, per device
         static bool done[64] = {};
@@ -299,6 +404,14 @@ int launch_rows(const SpmvArgs &a, int grid, size_t lds_bytes, hipStream_t strea
     return (int)hipGetLastError();
 }
 
+// Launch-shape overrides for tuning runs (0 = built-in default).  Not part of the public ABI.
+struct Tuning {
+    int block;      // threads per workgroup: 256, 512 or 1024
+    int depth;      // tiles in flight per wave: 2, 4 or 8
+    int wg_per_cu;  // workgroups launched per compute unit
+};
+Tuning g_tuning = {0, 0, 0};
+
 template <bool AXPBY>
 int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 {
@@ -312,16 +425,34 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     int rc = device_info(&info);
     if (rc != 0) return rc;
 
-    constexpr int BLOCK = 1024;
-    constexpr int WAVES = BLOCK / kWave;
-    int grid = (a.rows + WAVES - 1) / WAVES;
-    if (grid > info.compute_units) grid = info.compute_units;
+    const Tuning t = g_tuning;
+    const int block = t.block ? t.block : 1024;
+    const int depth = t.depth ? t.depth : 8;
+    const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
+    const int waves = block / kWave;
+    // at most one wave per tile: tiny matrices get a small grid
+    const long long n_tiles = (a.padded + kTile - 1) / kTile;
+    long long grid = (n_tiles + waves - 1) / waves;
+    if (grid > (long long)info.compute_units * wg_per_cu) grid = (long long)info.compute_units * wg_per_cu;
     if (grid < 1) grid = 1;
 
     const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
-    if (lds_need <= (size_t)info.max_lds_bytes)
-        return launch_rows<BLOCK, 4, true, AXPBY>(a, grid, lds_need, stream);
-    return launch_rows<BLOCK, 4, false, AXPBY>(a, grid, 0, stream);
+    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 8, false, AXPBY>(a, (int)grid, 0, stream);
+#define MACKO_CASE(B, D_) \
+    if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
+    MACKO_CASE(1024, 8)
+    if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
+        MACKO_CASE(1024, 2)
+        MACKO_CASE(1024, 4)
+        MACKO_CASE(512, 2)
+        MACKO_CASE(512, 4)
+        MACKO_CASE(512, 8)
+        MACKO_CASE(256, 2)
+        MACKO_CASE(256, 4)
+        MACKO_CASE(256, 8)
+    }
+#undef MACKO_CASE
+    return MACKO_E_INVALID_ARGUMENT;
 }
 
 int check_spmv_args(const void *values, const void *deltas, const int32_t *row_ptr, const void *x, void *y,
@@ -343,6 +474,12 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 }  // namespace
 }  // namespace macko
 
+// Tuning hook used by benchmark sweeps; see struct Tuning.
+extern "C" void macko_spmv_tune(int block, int depth, int wg_per_cu)
+{
+    macko::g_tuning = macko::Tuning{block, depth, wg_per_cu};
+}
+
 extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_ptr, const void *x,
                               void *y, int32_t rows, int32_t cols, int64_t padded_entries, void *stream)
 {
@@ -350,7 +487,8 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
     int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
-               rows,                cols,                padded_entries, 1.0f,          0.0f};
+               rows,                cols,                padded_entries, 1.0f,          0.0f,
+               0,                   0,                   0,              0,             0};
     return spmv_dispatch<false>(a, as_stream(stream));
 }
 
@@ -362,6 +500,7 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
-               rows,                cols,                padded_entries, alpha,         beta};
+               rows,                cols,                padded_entries, alpha,         beta,
+               0,                   0,                   0,              0,             0};
     return spmv_dispatch<true>(a, as_stream(stream));
 }
