@@ -63,7 +63,7 @@ def build_hip(verbose=False):
         _hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
         # keep the compiler from forming packed fp32 VALU ops (device pass; the host pass ignores it)
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wno-unused-command-line-argument",
+        "-Wno-unused-command-line-argument", "-Wno-inline-asm",
         f"-I{_INCLUDE}", f"-I{_CSRC}",
         *[os.path.join(_CSRC, s) for s in HIP_SOURCES],
         "-o", out,

@@ -74,4 +74,18 @@ __device__ __forceinline__ int wave_scan_max_inclusive(int x)
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
+// Compile-time loop: calls f(std::integral_constant<int, 0>{}) ... f(<N-1>{}) in order.
+template <int I>
+struct index_constant {
+    static constexpr int value = I;
+};
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(index_constant<I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 }  // namespace macko

@@ -28,7 +28,7 @@ namespace {
 constexpr int kLdsFront = 16;   // zero bytes in front of x in LDS (masked head entries read here)
 constexpr int kLdsBack = 64;    // zero bytes behind x (masked tail entries read here)
 constexpr int kTileShift = 9;   // log2(kTile)
-constexpr int kXRegs = 2;       // 16-byte pieces of x a thread carries in registers while staging
+constexpr int kXRegs = 2;       // 16-byte pieces of x a thread fetches with tracked loads
 
 struct SpmvArgs {
     const u32 *values;      // fp16 pairs
@@ -45,7 +45,17 @@ struct SpmvArgs {
     // does no 64-bit division: wave w starts at w*q + min(w, rem)
     u32 n_tiles, tiles_q, tiles_rem;
     u32 rows_q, rows_rem;
+#ifdef MACKO_SPMV_TRACE
+    long long *trace;  // 8 timestamps per wave (development builds only)
+#endif
 };
+
+#ifdef MACKO_SPMV_TRACE
+#define MACKO_STAMP(slot) \
+    do { if (a.trace && lane == 0) a.trace[(size_t)gw * 8 + (slot)] = (long long)__builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define MACKO_STAMP(slot) do { } while (0)
+#endif
 
 // First item of wave w when n items are dealt to the waves as evenly as possible.
 __device__ __forceinline__ u32 even_split(u32 w, u32 q, u32 rem) { return w * q + (w < rem ? w : rem); }
@@ -155,25 +165,199 @@ __device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= u
     d &= (1u << (4 * upto)) - 1;
 }
 
+// ---- loads whose completion is tracked by hand ---------------------------------------------
+// The tile ring, the row_ptr probe and the first pieces of x are fetched with inline-asm buffer
+// loads into FIXED physical VGPRs and awaited with explicit s_waitcnt vmcnt(N).  Vector-memory
+// loads complete in issue order, so "at most N loads outstanding" proves that every load older
+// than the N youngest has landed; N is always the number of tracked loads issued after the one
+// being awaited (loads or stores the compiler issues on its own can only make such a wait
+// longer, never too short).  The kernel is compiled with amdgpu_num_vgpr(kCompilerVgprs), which
+// keeps the register allocator below the fixed registers, so nothing else ever lives in them;
+// a `take` copies a landed slot into ordinary registers after its wait.  The byte offset goes
+// into the VGPR operand because only that operand takes part in the buffer's bounds check:
+// past-the-end addresses read as zero without touching memory, which is also how "no tile" is
+// encoded (kNoTile*).
+//
+// Register map (kCompilerVgprs = 78):  v78,v79 row_ptr probes; v80..v87 two 16-byte pieces of x;
+// v88.. ring: slot j keeps its values in v[88+4j : 91+4j] and its delta word in v[88+4D+j].
+
+constexpr int kCompilerVgprs = 78;
+constexpr u32 kNoTileValues = 0xfffff000u;  // beyond any values array (2P < 2^32 - 8192)
+constexpr u32 kNoTileDeltas = 0x7ffff000u;  // beyond any deltas array (P/2 < 2^30)
+
+__device__ __forceinline__ u32x4 make_buffer(const void *base, u32 bytes)
+{
+    const unsigned long long addr = reinterpret_cast<unsigned long long>(base);
+    u32x4 r;
+    r.x = uniform((int)(u32)addr);
+    r.y = uniform((int)((u32)(addr >> 32) & 0xffffu));
+    r.z = uniform((int)bytes);
+    r.w = 0x00020000u;
+    return r;
+}
+
+#define MACKO_FIXED_CLOBBERS_16 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167"
+#define MACKO_FIXED_CLOBBERS_8 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127"
+#define MACKO_FIXED_CLOBBERS_4 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107"
+
+// row_ptr probe k (k = 0, 1) -> v78 + k
+template <int K>
+__device__ __forceinline__ void probe_issue(u32 byte_offset, const u32x4 &buffer)
+{
+    if (K == 0) asm volatile("buffer_load_dword v78, %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer) : "memory", "v78");
+    if (K == 1) asm volatile("buffer_load_dword v79, %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer) : "memory", "v79");
+}
+template <int K, int N>
+__device__ __forceinline__ int probe_take()
+{
+    int w;
+    if (K == 0) asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, v78" : "=v"(w) : "n"(N) : "memory");
+    if (K == 1) asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, v79" : "=v"(w) : "n"(N) : "memory");
+    return w;
+}
+
+// piece j of x (j = 0, 1) -> v[80+4j : 83+4j]
+template <int J>
+__device__ __forceinline__ void xpiece_issue(u32 byte_offset, const u32x4 &buffer)
+{
+    if (J == 0)
+        asm volatile("buffer_load_dwordx4 v[80:83], %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer)
+                     : "memory", "v80", "v81", "v82", "v83");
+    if (J == 1)
+        asm volatile("buffer_load_dwordx4 v[84:87], %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer)
+                     : "memory", "v84", "v85", "v86", "v87");
+}
+template <int J, int N>
+__device__ __forceinline__ u32x4 xpiece_take()
+{
+    u32x4 v;
+    if (J == 0)
+        asm volatile("s_waitcnt vmcnt(%4)\n\tv_mov_b32 %0, v80\n\tv_mov_b32 %1, v81\n\tv_mov_b32 %2, v82\n\tv_mov_b32 %3, v83"
+                     : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w) : "n"(N) : "memory");
+    if (J == 1)
+        asm volatile("s_waitcnt vmcnt(%4)\n\tv_mov_b32 %0, v84\n\tv_mov_b32 %1, v85\n\tv_mov_b32 %2, v86\n\tv_mov_b32 %3, v87"
+                     : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w) : "n"(N) : "memory");
+    return v;
+}
+
+// ring slot J of a D-deep ring: issue both loads / wait and copy out
+#define MACKO_RING_ISSUE(VREGS, DREG, CLOBBERS)                                                            \
+    asm volatile("buffer_load_dwordx4 " VREGS ", %0, %2, 0 offen\n\tbuffer_load_dword " DREG ", %1, %3, 0 offen" \
+                 ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
+                 : "memory", CLOBBERS)
+#define MACKO_RING_TAKE(A, B, C, E, DREG)                                                                      \
+    asm volatile("s_waitcnt vmcnt(%5)\n\tv_mov_b32 %0, " A "\n\tv_mov_b32 %1, " B "\n\tv_mov_b32 %2, " C          \
+                 "\n\tv_mov_b32 %3, " E "\n\tv_mov_b32 %4, " DREG                                               \
+                 : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w), "=v"(d) : "n"(N) : "memory")
+
+template <int D, int J>
+__device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
+                                           const u32x4 &buf_deltas)
+{
+    static_assert(D == 4 || D == 8 || D == 16, "ring depth");
+    if (D == 4 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v104", MACKO_FIXED_CLOBBERS_4);
+    if (D == 4 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v105", MACKO_FIXED_CLOBBERS_4);
+    if (D == 4 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v106", MACKO_FIXED_CLOBBERS_4);
+    if (D == 4 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v107", MACKO_FIXED_CLOBBERS_4);
+    if (D == 8 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v120", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v121", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v122", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v123", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 4) MACKO_RING_ISSUE("v[104:107]", "v124", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 5) MACKO_RING_ISSUE("v[108:111]", "v125", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 6) MACKO_RING_ISSUE("v[112:115]", "v126", MACKO_FIXED_CLOBBERS_8);
+    if (D == 8 && J == 7) MACKO_RING_ISSUE("v[116:119]", "v127", MACKO_FIXED_CLOBBERS_8);
+    if (D == 16 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v152", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v153", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v154", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v155", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 4) MACKO_RING_ISSUE("v[104:107]", "v156", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 5) MACKO_RING_ISSUE("v[108:111]", "v157", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 6) MACKO_RING_ISSUE("v[112:115]", "v158", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 7) MACKO_RING_ISSUE("v[116:119]", "v159", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 8) MACKO_RING_ISSUE("v[120:123]", "v160", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 9) MACKO_RING_ISSUE("v[124:127]", "v161", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 10) MACKO_RING_ISSUE("v[128:131]", "v162", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 11) MACKO_RING_ISSUE("v[132:135]", "v163", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 12) MACKO_RING_ISSUE("v[136:139]", "v164", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 13) MACKO_RING_ISSUE("v[140:143]", "v165", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 14) MACKO_RING_ISSUE("v[144:147]", "v166", MACKO_FIXED_CLOBBERS_16);
+    if (D == 16 && J == 15) MACKO_RING_ISSUE("v[148:151]", "v167", MACKO_FIXED_CLOBBERS_16);
+}
+
+template <int D, int J, int N>
+__device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
+{
+    if (D == 4 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v104");
+    if (D == 4 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v105");
+    if (D == 4 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v106");
+    if (D == 4 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v107");
+    if (D == 8 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v120");
+    if (D == 8 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v121");
+    if (D == 8 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v122");
+    if (D == 8 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v123");
+    if (D == 8 && J == 4) MACKO_RING_TAKE("v104", "v105", "v106", "v107", "v124");
+    if (D == 8 && J == 5) MACKO_RING_TAKE("v108", "v109", "v110", "v111", "v125");
+    if (D == 8 && J == 6) MACKO_RING_TAKE("v112", "v113", "v114", "v115", "v126");
+    if (D == 8 && J == 7) MACKO_RING_TAKE("v116", "v117", "v118", "v119", "v127");
+    if (D == 16 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v152");
+    if (D == 16 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v153");
+    if (D == 16 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v154");
+    if (D == 16 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v155");
+    if (D == 16 && J == 4) MACKO_RING_TAKE("v104", "v105", "v106", "v107", "v156");
+    if (D == 16 && J == 5) MACKO_RING_TAKE("v108", "v109", "v110", "v111", "v157");
+    if (D == 16 && J == 6) MACKO_RING_TAKE("v112", "v113", "v114", "v115", "v158");
+    if (D == 16 && J == 7) MACKO_RING_TAKE("v116", "v117", "v118", "v119", "v159");
+    if (D == 16 && J == 8) MACKO_RING_TAKE("v120", "v121", "v122", "v123", "v160");
+    if (D == 16 && J == 9) MACKO_RING_TAKE("v124", "v125", "v126", "v127", "v161");
+    if (D == 16 && J == 10) MACKO_RING_TAKE("v128", "v129", "v130", "v131", "v162");
+    if (D == 16 && J == 11) MACKO_RING_TAKE("v132", "v133", "v134", "v135", "v163");
+    if (D == 16 && J == 12) MACKO_RING_TAKE("v136", "v137", "v138", "v139", "v164");
+    if (D == 16 && J == 13) MACKO_RING_TAKE("v140", "v141", "v142", "v143", "v165");
+    if (D == 16 && J == 14) MACKO_RING_TAKE("v144", "v145", "v146", "v147", "v166");
+    if (D == 16 && J == 15) MACKO_RING_TAKE("v148", "v149", "v150", "v151", "v167");
+}
 template <int BLOCK, int D, bool X_LDS, bool AXPBY>
-__global__ void __launch_bounds__(BLOCK) spmv_stream_kernel(const SpmvArgs a)
+__global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
+spmv_stream_kernel(const SpmvArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int WAVES = BLOCK / kWave;
+    constexpr int kTileLoads = 2 * D;  // tracked loads per full ring
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = uniform(tid >> 6);
     const u32 n_waves = gridDim.x * WAVES;
     const u32 gw = blockIdx.x * WAVES + wave;
+    MACKO_STAMP(0);
 
     const u32 nt_lo = even_split(gw, a.tiles_q, a.tiles_rem);
     const u32 nt_hi = even_split(gw + 1, a.tiles_q, a.tiles_rem);
 
-    // Loads are issued in the order probe, x, tiles; they complete in that order, so each
-    // consumer below waits only for what was issued before its own data.
+    const u32x4 buf_values = make_buffer(a.values, (u32)(a.padded * 2));
+    const u32x4 buf_deltas = make_buffer(a.deltas, (u32)(a.padded / 2));
+    const u32x4 buf_rows = make_buffer(a.row_ptr, ((u32)a.rows + 1) * 4);
+    const __amdgpu_buffer_rsrc_t rs_x =
+        __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.cols * 2, 0x00020000);
+    (void)rs_x;
+    const u32 lane16 = (u32)lane * 16, lane4 = (u32)lane * 4;
 
-    // ---- 1. row_ptr probe ---------------------------------------------------------------------
-    int target[2], base[2], window[2];
+    // ---- 1. x: everything beyond the two register pieces per thread, and unaligned or odd-length
+    //         x, is copied first (ordinary loads; done before any tracked load is issued) ---------
+    const bool x_vec = (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+    const int x_nvec = x_vec ? a.cols >> 3 : 0;
+    if (X_LDS) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
+        for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
+        for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
+        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
+        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
+    }
+
+    // ---- 2. tracked loads, oldest first: row_ptr probes, x pieces ------------------------------------
+    // probes: 64 consecutive row_ptr values around where my first / last row should be
+    int target[2], base[2];
     {
         const unsigned long long t0 = (unsigned long long)nt_lo << kTileShift;
         const unsigned long long t1 = (unsigned long long)nt_hi << kTileShift;
@@ -181,67 +365,52 @@ __global__ void __launch_bounds__(BLOCK) spmv_stream_kernel(const SpmvArgs a)
         target[1] = t1 > 0x7fffffffull ? 0x7fffffff : (int)t1;
         base[0] = probe_base((int)even_split(gw, a.rows_q, a.rows_rem), a.rows);
         base[1] = probe_base((int)even_split(gw + 1, a.rows_q, a.rows_rem), a.rows);
-        window[0] = load_row_window(a.row_ptr, a.rows, base[0], lane);
-        window[1] = load_row_window(a.row_ptr, a.rows, base[1], lane);
+        int i0 = base[0] + lane, i1 = base[1] + lane;
+        i0 = i0 <= a.rows ? i0 : a.rows;
+        i1 = i1 <= a.rows ? i1 : a.rows;
+        probe_issue<0>((u32)i0 * 4, buf_rows);
+        probe_issue<1>((u32)i1 * 4, buf_rows);
     }
-
-    // ---- 2. x: the first pieces travel through registers ---------------------------------------
-    const bool x_vec = (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
-    const int x_nvec = x_vec ? a.cols >> 3 : 0;
-    u32x4 xr[kXRegs];
+    const u32x4 buf_x = make_buffer(a.x, (u32)x_nvec * 16);  // past the end reads as zero
     if (X_LDS) {
-#pragma unroll
-        for (int j = 0; j < kXRegs; ++j) {
-            const int i = tid + j * BLOCK;
-            xr[j] = (u32x4){0, 0, 0, 0};
-            if (i < x_nvec) xr[j] = reinterpret_cast<const u32x4 *>(a.x)[i];
-        }
+        xpiece_issue<0>((u32)tid * 16, buf_x);
+        xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
+    auto issue_slot = [&](auto slot, u32 tile, bool fetch) {
+        constexpr int J = decltype(slot)::value;
+        ring_issue<D, J>(lane16 + (fetch ? tile << (kTileShift + 1) : kNoTileValues),
+                         lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas);
+    };
+    MACKO_STAMP(1);
 
-    // ---- 3. the first D tiles of my nominal range -----------------------------------------------
-    const __amdgpu_buffer_rsrc_t rs_values =
-        __builtin_amdgcn_make_buffer_rsrc((void *)a.values, 0, (int)(u32)(a.padded * 2), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rs_deltas =
-        __builtin_amdgcn_make_buffer_rsrc((void *)a.deltas, 0, (int)(a.padded / 2), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rs_x =
-        __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.cols * 2, 0x00020000);
-    (void)rs_x;
-    u32x4 v[D];
-    u32 d[D];
-#pragma unroll
-    for (int j = 0; j < D; ++j) {
-        const u32 tile = nt_lo + j;
-        v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_values, lane * 16, (int)(tile << (kTileShift + 1)), 0);
-        d[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_deltas, lane * 4, (int)(tile << (kTileShift - 1)), 0);
-    }
-
-    // ---- 4. which rows are mine -------------------------------------------------------------------
+    // ---- 3. which rows are mine -----------------------------------------------------------------------
+    constexpr int kXLoads = X_LDS ? kXRegs : 0;
+    int window[2];
+    window[0] = probe_take<0, kXLoads + 1>();
+    window[1] = probe_take<1, kXLoads>();
     int range[2];
     wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
     if (gw == n_waves - 1) range[1] = a.rows;
     if (nt_lo == nt_hi) range[1] = range[0];  // no nominal tiles: owns nothing
     const int row_first = uniform(range[0]);
     const int row_last = uniform(range[1]);
+    MACKO_STAMP(2);
 
-    // ---- 5. x into LDS ------------------------------------------------------------------------------
+    // ---- 4. x pieces into LDS ---------------------------------------------------------------------------
     if (X_LDS) {
-        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
-        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
-#pragma unroll
-        for (int j = 0; j < kXRegs; ++j) {
-            const int i = tid + j * BLOCK;
-            if (i < x_nvec) d4[i] = xr[j];
-        }
-        for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
-        for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(lds + kLdsFront);
+        const u32x4 x0 = xpiece_take<0, 1>();
+        if (tid < x_nvec) d4[tid] = x0;
+        const u32x4 x1 = xpiece_take<1, 0>();
+        if (tid + BLOCK < x_nvec) d4[tid + BLOCK] = x1;
+        MACKO_STAMP(3);
         __syncthreads();
     }
+    MACKO_STAMP(4);
 
     if (row_first >= row_last) return;
 
-    // ---- 6. stream --------------------------------------------------------------------------------
+    // ---- 6. stream ----------------------------------------------------------------------------------
     // window of row_ptr values: lane i holds row_ptr[win_base + i]
     int win_base = base[0];
     int win = window[0];
@@ -285,78 +454,96 @@ __global__ void __launch_bounds__(BLOCK) spmv_stream_kernel(const SpmvArgs a)
 
     float acc0 = 0.f, acc1 = 0.f;
     int carry = 0;  // nibble sum of the current row so far
+    typedef __attribute__((address_space(3))) const uint16_t *lds_u16_ptr;
+    const u32 lds_base = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+    MACKO_STAMP(5);
 
-    for (u32 tile0 = nt_lo; tile0 < last_tile; tile0 += D) {
+    // One segment pass: entries [pos, seg_end) of tile `tb`, all in row r.
+    auto tile_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end) {
+#if defined(MACKO_EXP_NO_COMPUTE)
+        acc0 += __builtin_bit_cast(float, (vj.x ^ vj.y ^ vj.z ^ vj.w ^ dj) & 0x3fffffffu);
+        return;
+#endif
+        const int rel0 = pos - tb;
+        const int rel1 = seg_end - tb;
+        u32x4 vv = vj;
+        u32 dd = dj;
+        bool active = true;
+        if (rel0 != 0 || rel1 != kTile) {  // not the whole tile (wave-uniform test)
+            const int l0 = rel0 >> 3, q0 = rel0 & 7;
+            const int l1 = (rel1 - 1) >> 3, q1 = rel1 & 7;
+            active = lane >= l0 && lane <= l1;
+            if (!active) dd = 0;
+            if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
+            if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
+        }
+        const int s = (int)__builtin_amdgcn_udot8(dd, 0x11111111u, 0u, false);
+        const int incl = wave_scan_inclusive(s);
+        // LDS byte address of x[col] for entry 0 of this chunk, before its own nibble:
+        // kLdsFront + 2 * (entry index in the row + nibbles before it); tb + 8*lane - e0 >= -7 for an
+        // active lane, so it stays positive.  The wave-uniform part is folded on the scalar unit.
+        const u32 uniform_part = lds_base + (u32)(kLdsFront + 2 * (tb - e0 + carry));
+        const u32 addr0 = ((u32)(incl - s) << 1) + (lane16 + uniform_part);
+        carry += __builtin_amdgcn_readlane(incl, kWave - 1);
+        if (active) {
+            const u32 m[8] = {0x2u, 0x22u, 0x222u, 0x2222u, 0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
 #pragma unroll
-        for (int j = 0; j < D; ++j) {
-            const u32 tile = tile0 + j;
-            if (tile >= last_tile) continue;  // wave-uniform
-            const u32x4 vj = v[j];
-            const u32 dj = d[j];
-            if (tile + D < last_tile) {  // refill this ring slot
-                v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_values, lane * 16,
-                                                              (int)((tile + D) << (kTileShift + 1)), 0);
-                d[j] = __builtin_amdgcn_raw_buffer_load_b32(rs_deltas, lane * 4,
-                                                             (int)((tile + D) << (kTileShift - 1)), 0);
+            for (int k = 0; k < 8; ++k) {
+                const u32 addr = __builtin_amdgcn_udot8(dd, m[k], addr0, false);
+                uint16_t xb;
+#if defined(MACKO_EXP_NO_GATHER)
+                xb = (uint16_t)(addr & 0x3fffu);
+#else
+                if (X_LDS) {
+                    // addr already carries the LDS base, so this is a bare ds_read_u16 with an
+                    // immediate offset
+                    xb = *reinterpret_cast<lds_u16_ptr>((u32)(addr + 2 * k));
+                } else {
+                    int o = (int)addr + 2 * k - kLdsFront;
+                    const int omax = 2 * a.cols - 2;
+                    o = o < 0 ? 0 : (o > omax ? omax : o);
+                    xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
+                }
+#endif
+                const u32 w = vv[k >> 1];
+                const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+                if (k & 1)
+                    acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
+                else
+                    acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
             }
-            if (tile < first_tile) continue;  // fetched on speculation, belongs to the previous wave
+        }
+    };
+
+    // Fill the ring with my first D tiles, then: take a slot, process it, refill it.  Every step
+    // issues exactly two loads (a "no tile" address once the range is exhausted), so a slot's
+    // loads are always followed by those of the D - 1 other slots when it is awaited.
+    static_for<D>([&](auto slot) {
+        constexpr int J = decltype(slot)::value;
+        issue_slot(slot, first_tile + J, first_tile + J < last_tile);
+    });
+    for (u32 tile0 = first_tile; tile0 < last_tile; tile0 += D) {
+        static_for<D>([&](auto slot) {
+            constexpr int J = decltype(slot)::value;
+            const u32 tile = tile0 + J;
+            if (tile >= last_tile) return;  // wave-uniform; nothing is awaited or issued after this
+            u32x4 vj;
+            u32 dj;
+            ring_take<D, J, kTileLoads - 2>(vj, dj);
+            issue_slot(slot, tile + D, tile + D < last_tile);  // refill at once: the copy is out
             const int tb = (int)(tile << kTileShift);
             const int lim = tb + kTile < s_end ? tb + kTile : s_end;
             int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
             while (pos < lim) {
                 const int seg_end = e1 < lim ? e1 : lim;
-                // ---- one pass over the segment [pos, seg_end) of row r ----
-                const int rel0 = pos - tb;
-                const int rel1 = seg_end - tb;
-                u32x4 vv = vj;
-                u32 dd = dj;
-                bool active = true;
-                if (rel0 != 0 || rel1 != kTile) {  // not the whole tile (wave-uniform test)
-                    const int l0 = rel0 >> 3, q0 = rel0 & 7;
-                    const int l1 = (rel1 - 1) >> 3, q1 = rel1 & 7;
-                    active = lane >= l0 && lane <= l1;
-                    if (!active) dd = 0;
-                    if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
-                    if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
-                }
-                const int s = (int)__builtin_amdgcn_udot8(dd, 0x11111111u, 0u, false);
-                const int incl = wave_scan_inclusive(s);
-                const int excl = incl - s + carry;
-                carry += __builtin_amdgcn_readlane(incl, kWave - 1);
-                if (active) {
-                    // LDS byte address of x[col] for entry 0 of this chunk, before its own nibble;
-                    // tb + 8*lane - e0 >= -7 for an active lane, so this stays positive
-                    const u32 addr0 = (u32)(kLdsFront + 2 * (tb + 8 * lane - e0 + excl));
-                    const u32 m[8] = {0x2u,     0x22u,     0x222u,     0x2222u,
-                                      0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const u32 addr = __builtin_amdgcn_udot8(dd, m[k], addr0, false);
-                        uint16_t xb;
-                        if (X_LDS) {
-                            xb = *reinterpret_cast<const uint16_t *>(lds + addr + 2 * k);
-                        } else {
-                            int o = (int)addr + 2 * k - kLdsFront;
-                            const int omax = 2 * a.cols - 2;
-                            o = o < 0 ? 0 : (o > omax ? omax : o);
-                            xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
-                        }
-                        const u32 w = vv[k >> 1];
-                        const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
-                        if (k & 1)
-                            acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
-                        else
-                            acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
-                    }
-                }
-                // ---- row finished? ----
-                if (seg_end == e1) {
+                tile_pass(vj, dj, tb, pos, seg_end);
+                if (seg_end == e1) {  // row finished
                     store_row(r, wave_sum(acc0 + acc1));
                     acc0 = acc1 = 0.f;
                     carry = 0;
                     do {  // next non-empty owned row; empty ones get their zero on the way
                         ++r;
-                        if (r >= row_last) break;  // then seg_end == s_end == lim and both loops end
+                        if (r >= row_last) break;  // then seg_end == s_end == lim and all loops end
                         slide_window(r);
                         e0 = row_start(r);
                         e1 = row_start(r + 1);
@@ -365,8 +552,9 @@ __global__ void __launch_bounds__(BLOCK) spmv_stream_kernel(const SpmvArgs a)
                 }
                 pos = seg_end;
             }
-        }
+        });
     }
+    MACKO_STAMP(6);
 }
 
 // y[r] = 0 (or beta*y[r]) for matrices without stored entries.
@@ -407,7 +595,7 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 // Launch-shape overrides for tuning runs (0 = built-in default).  Not part of the public ABI.
 struct Tuning {
     int block;      // threads per workgroup: 256, 512 or 1024
-    int depth;      // tiles in flight per wave: 2, 4 or 8
+    int depth;      // tiles in flight per wave: 4, 8 or 16 (16 only with 256 or 512 threads)
     int wg_per_cu;  // workgroups launched per compute unit
 };
 Tuning g_tuning = {0, 0, 0};
@@ -442,14 +630,13 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
     MACKO_CASE(1024, 8)
     if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
-        MACKO_CASE(1024, 2)
         MACKO_CASE(1024, 4)
-        MACKO_CASE(512, 2)
         MACKO_CASE(512, 4)
         MACKO_CASE(512, 8)
-        MACKO_CASE(256, 2)
+        MACKO_CASE(512, 16)
         MACKO_CASE(256, 4)
         MACKO_CASE(256, 8)
+        MACKO_CASE(256, 16)
     }
 #undef MACKO_CASE
     return MACKO_E_INVALID_ARGUMENT;
@@ -460,7 +647,7 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 {
     if (rows < 0 || cols < 0 || padded < 0) return MACKO_E_INVALID_ARGUMENT;
     if (padded % kChunk != 0) return MACKO_E_INVALID_ARGUMENT;
-    if (padded >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
+    if (padded >= (1ll << 31) - 8192) return MACKO_E_INVALID_ARGUMENT;
     if (rows > 0 && (row_ptr == nullptr || y == nullptr)) return MACKO_E_INVALID_ARGUMENT;
     if (padded > 0 && (values == nullptr || deltas == nullptr || x == nullptr || cols == 0))
         return MACKO_E_INVALID_ARGUMENT;
@@ -473,6 +660,11 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 
 }  // namespace
 }  // namespace macko
+
+#ifdef MACKO_SPMV_TRACE
+static long long *g_trace = nullptr;
+extern "C" void macko_spmv_set_trace(long long *device_buffer) { g_trace = device_buffer; }
+#endif
 
 // Tuning hook used by benchmark sweeps; see struct Tuning.
 extern "C" void macko_spmv_tune(int block, int depth, int wg_per_cu)
@@ -489,6 +681,9 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
                0,                   0,                   0,              0,             0};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = g_trace;
+#endif
     return spmv_dispatch<false>(a, as_stream(stream));
 }
 
@@ -502,5 +697,8 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
                0,                   0,                   0,              0,             0};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = nullptr;
+#endif
     return spmv_dispatch<true>(a, as_stream(stream));
 }
