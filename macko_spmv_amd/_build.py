@@ -10,9 +10,11 @@ directory -- the same variable the upstream package reads for its JIT cache
 Run `python -m macko_spmv_amd._build` to (re)build both.
 """
 import os
+import re
 import shutil
 import subprocess
 import sys
+import tempfile
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_PKG)
@@ -57,18 +59,64 @@ def _run(cmd, verbose):
         print(proc.stdout, flush=True)
 
 
+_DEVICE_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17",
+    # keep the compiler from forming packed fp32 VALU ops (device pass; the host pass ignores it)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
+    f"-I{_INCLUDE}", f"-I{_CSRC}",
+]
+
+# The SpMV kernel keeps its in-flight loads in fixed VGPRs from this one up (kCompilerVgprs in
+# macko_spmv.hip); compiler-generated code must stay below it.
+FIXED_VGPR_BASE = 78
+
+
+def verify_fixed_registers(verbose=False):
+    """Compile macko_spmv.hip to assembly and check that, outside the hand-written asm blocks, no
+    instruction of any spmv_stream_kernel touches a VGPR >= FIXED_VGPR_BASE."""
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "macko_spmv.s")
+        _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, "macko_spmv.hip"), "-o", asm],
+             verbose)
+        text = open(asm).read().splitlines()
+    kernel = None
+    in_asm = False
+    checked = 0
+    for line in text:
+        m = re.match(r"^(_Z\S*spmv_stream_kernel\S*):", line)
+        if m:
+            kernel, in_asm = m.group(1), False
+            checked += 1
+            continue
+        if kernel is None:
+            continue
+        if "s_endpgm" in line:
+            kernel = None
+        elif "#ASMSTART" in line:
+            in_asm = True
+        elif "#ASMEND" in line:
+            in_asm = False
+        elif not in_asm:
+            code = line.split(";")[0]
+            regs = [int(b) for _, b in re.findall(r"\bv\[(\d+):(\d+)\]", code)]
+            regs += [int(a) for a in re.findall(r"\bv(\d+)\b", code)]
+            if regs and max(regs) >= FIXED_VGPR_BASE:
+                raise RuntimeError(f"compiler-generated code touches a fixed VGPR in {kernel}: {line.strip()}")
+    if checked == 0:
+        raise RuntimeError("no spmv_stream_kernel found in the assembly; the register check is stale")
+    return checked
+
+
 def build_hip(verbose=False):
     out, _ = lib_paths()
     cmd = [
-        _hipcc(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
-        # keep the compiler from forming packed fp32 VALU ops (device pass; the host pass ignores it)
-        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wno-unused-command-line-argument", "-Wno-inline-asm",
-        f"-I{_INCLUDE}", f"-I{_CSRC}",
+        _hipcc(), *_DEVICE_FLAGS, "-fPIC", "-shared",
         *[os.path.join(_CSRC, s) for s in HIP_SOURCES],
         "-o", out,
     ]
     _run(cmd, verbose)
+    verify_fixed_registers(verbose)
     return out
 
 

@@ -1,17 +1,16 @@
 // MACKO fp16 sparse matrix-vector product for gfx950 (wave64).
 //
-// Data movement.  The value and delta arrays are cut into fixed tiles of 512 entries (one
-// 128-bit value load and one 32-bit delta load per lane).  The launch has W waves; wave w
-// streams the tiles [w*NT/W, (w+1)*NT/W) and a little beyond, keeping D tiles in flight in a
-// register ring.  Because tile positions do not depend on row_ptr, the first D loads are issued
-// at the top of the kernel, together with the row_ptr probe and the copy of x into LDS: one
-// memory latency, not a chain of them, sits in front of the first multiply-add.
+// Row ownership.  The value and delta arrays are cut into fixed tiles of 512 entries (one
+// 128-bit value load and one 32-bit delta load per lane).  The launch has W waves; wave w owns
+// the rows whose first entry index lies inside the tile range [w*NT/W, (w+1)*NT/W): contiguous
+// whole rows, balanced by stored entries.  It finds them with a 64-wide probe of row_ptr placed
+// by an arithmetic guess (one memory round trip when rows carry similar entry counts, 64-ary
+// search rounds otherwise).  No row is shared between waves, so there is no cross-wave
+// reduction, no atomics and no scratch memory.
 //
-// Row ownership.  Wave w owns the rows whose first entry index lies inside its nominal tile
-// range (contiguous whole rows, balanced by stored entries, found with a 64-wide search of
-// row_ptr).  It walks from the tile holding its first owned entry to the tile holding its last,
-// which overlaps the neighbours' nominal ranges by at most one row.  No row is shared between
-// waves, so there is no cross-wave reduction, no atomics and no scratch memory.
+// Data movement.  While the probe is in flight the workgroup copies x into LDS.  Each wave then
+// streams the tiles that hold its rows through a ring of D register slots (hand-tracked loads,
+// see below): take a slot, refill it with the tile D ahead, process.
 //
 // Per tile, the entries of one row form a segment [first lane/entry, last lane/entry]; each
 // segment takes one pass: mask, DPP prefix sum of per-lane nibble sums, v_dot8_u32_u4 for the
@@ -41,9 +40,9 @@ struct SpmvArgs {
     long long padded;       // P
     float alpha;
     float beta;
-    // split of tiles and rows over the launch's waves, precomputed on the host so the kernel
-    // does no 64-bit division: wave w starts at w*q + min(w, rem)
-    u32 n_tiles, tiles_q, tiles_rem;
+    // split of the P stored entries and of the rows over the launch's waves, precomputed on the
+    // host so the kernel does no 64-bit division: wave w starts at w*q + min(w, rem)
+    u32 entries_q, entries_rem;
     u32 rows_q, rows_rem;
 #ifdef MACKO_SPMV_TRACE
     long long *trace;  // 8 timestamps per wave (development builds only)
@@ -331,8 +330,6 @@ spmv_stream_kernel(const SpmvArgs a)
     const u32 gw = blockIdx.x * WAVES + wave;
     MACKO_STAMP(0);
 
-    const u32 nt_lo = even_split(gw, a.tiles_q, a.tiles_rem);
-    const u32 nt_hi = even_split(gw + 1, a.tiles_q, a.tiles_rem);
 
     const u32x4 buf_values = make_buffer(a.values, (u32)(a.padded * 2));
     const u32x4 buf_deltas = make_buffer(a.deltas, (u32)(a.padded / 2));
@@ -359,10 +356,8 @@ spmv_stream_kernel(const SpmvArgs a)
     // probes: 64 consecutive row_ptr values around where my first / last row should be
     int target[2], base[2];
     {
-        const unsigned long long t0 = (unsigned long long)nt_lo << kTileShift;
-        const unsigned long long t1 = (unsigned long long)nt_hi << kTileShift;
-        target[0] = t0 > 0x7fffffffull ? 0x7fffffff : (int)t0;
-        target[1] = t1 > 0x7fffffffull ? 0x7fffffff : (int)t1;
+        target[0] = (int)even_split(gw, a.entries_q, a.entries_rem);  // < P < 2^31
+        target[1] = (int)even_split(gw + 1, a.entries_q, a.entries_rem);
         base[0] = probe_base((int)even_split(gw, a.rows_q, a.rows_rem), a.rows);
         base[1] = probe_base((int)even_split(gw + 1, a.rows_q, a.rows_rem), a.rows);
         int i0 = base[0] + lane, i1 = base[1] + lane;
@@ -390,8 +385,25 @@ spmv_stream_kernel(const SpmvArgs a)
     window[1] = probe_take<1, kXLoads>();
     int range[2];
     wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
+    // Cut at the row start NEAREST to the target rather than the first one at or after it: with
+    // rows of similar length every wave then gets the same number of rows.
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int rr = range[k];
+        if (rr > 0 && rr <= a.rows) {
+            int after, before;
+            if (rr - 1 >= base[k] && rr <= base[k] + 63) {
+                after = __builtin_amdgcn_readlane(window[k], rr - base[k]);
+                before = __builtin_amdgcn_readlane(window[k], rr - 1 - base[k]);
+            } else {
+                after = uniform(a.row_ptr[rr]);
+                before = uniform(a.row_ptr[rr - 1]);
+            }
+            if (target[k] - before < after - target[k]) range[k] = rr - 1;
+        }
+    }
+    if (gw == 0) range[0] = 0;
     if (gw == n_waves - 1) range[1] = a.rows;
-    if (nt_lo == nt_hi) range[1] = range[0];  // no nominal tiles: owns nothing
     const int row_first = uniform(range[0]);
     const int row_last = uniform(range[1]);
     MACKO_STAMP(2);
@@ -570,9 +582,8 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
     auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
-    a.n_tiles = (u32)((a.padded + kTile - 1) >> kTileShift);
-    a.tiles_q = a.n_tiles / n_waves;
-    a.tiles_rem = a.n_tiles % n_waves;
+    a.entries_q = (u32)(a.padded / n_waves);
+    a.entries_rem = (u32)(a.padded % n_waves);
     a.rows_q = (u32)a.rows / n_waves;
     a.rows_rem = (u32)a.rows % n_waves;
     if (lds_bytes > 64 * 1024) {
@@ -615,7 +626,7 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 
     const Tuning t = g_tuning;
     const int block = t.block ? t.block : 1024;
-    const int depth = t.depth ? t.depth : 8;
+    const int depth = t.depth ? t.depth : 4;
     const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
     const int waves = block / kWave;
     // at most one wave per tile: tiny matrices get a small grid
@@ -625,12 +636,12 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     if (grid < 1) grid = 1;
 
     const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
-    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 8, false, AXPBY>(a, (int)grid, 0, stream);
+    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 4, false, AXPBY>(a, (int)grid, 0, stream);
 #define MACKO_CASE(B, D_) \
     if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
-    MACKO_CASE(1024, 8)
+    MACKO_CASE(1024, 4)
     if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
-        MACKO_CASE(1024, 4)
+        MACKO_CASE(1024, 8)
         MACKO_CASE(512, 4)
         MACKO_CASE(512, 8)
         MACKO_CASE(512, 16)
@@ -680,7 +691,7 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = g_trace;
 #endif
@@ -696,7 +707,7 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
