@@ -29,6 +29,26 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008)]
 DENSITIES = [0.1, 0.2, 0.3, 0.5, 0.7, 0.9]
+LARGE_SHAPES = [(28672, 8192), (8192, 28672), (12288, 49152), (49152, 12288)]
+LARGE_DENSITIES = [0.1, 0.3, 0.5]
+
+# HBM bytes per launch of spmv_stream_kernel, averaged over the 18 launches of one step of the
+# default workload: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, each scaled by what the
+# same counter reports for calibration_copy_kernel on 256 MiB (factors 0.5000 and 1.0000).  Source:
+# profiles/spmv_stream_kernel_llama_shapes_hbm_traffic.md.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 42.83e6}
+
+WORKLOADS = {
+    "llama": "configs[1]: Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as fp16 SpMV, per-row "
+             "magnitude pruning, density in {0.1,0.2,0.3,0.5,0.7,0.9}; one step = one multiply of each of the "
+             "18 (shape, density) pairs, replayed from a HIP graph",
+    "large": "configs[2]: 28672x8192, 8192x28672, 12288x49152, 49152x12288 as fp16 SpMV, unstructured "
+             "Bernoulli masks at density 0.1, 0.3, 0.5; one step = one multiply of each of the 12 pairs, "
+             "replayed from a HIP graph",
+    "skew": "configs[3]: 14336x4096 fp16, per-row density from a power law (alpha 1.5) clipped to [0.01, 0.95] "
+            "with mean 0.3, all-zero rows and a 40-column zero gap in every row, next to a uniform Bernoulli "
+            "0.3 matrix of the same shape; one step = one multiply of each, replayed from a HIP graph",
+}
 
 
 def log(*a):
@@ -56,6 +76,53 @@ def make_pruned(torch, rows, cols, density, seed):
         W = W * mask
     x = torch.randn((cols,), device="cuda", dtype=torch.float32, generator=g).to(torch.float16)
     return W.contiguous(), x
+
+
+def make_bernoulli(torch, rows, cols, density, seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    W = (torch.randn((rows, cols), device="cuda", dtype=torch.float32, generator=g) * 0.02).to(torch.float16)
+    W = W * (torch.rand((rows, cols), device="cuda", generator=g) < density)
+    x = torch.randn((cols,), device="cuda", dtype=torch.float32, generator=g).to(torch.float16)
+    return W.contiguous(), x
+
+
+def make_skewed(torch, rows, cols, seed, mean_density=0.3, alpha=1.5, lo=0.01, hi=0.95, gap=40, zero_every=97):
+    """Per-row density ~ lo * Pareto(alpha), clipped to [lo, hi] and rescaled towards the mean; every
+    97th row all zero; a run of `gap` zero columns in every row."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    u = torch.rand((rows,), device="cuda", generator=g)
+    d = (lo * (1.0 - u) ** (-1.0 / alpha)).clamp(lo, hi)
+    for _ in range(20):
+        d = (d * (mean_density / d.mean())).clamp(lo, hi)
+    W = (torch.randn((rows, cols), device="cuda", dtype=torch.float32, generator=g) * 0.02).to(torch.float16)
+    W = W * (torch.rand((rows, cols), device="cuda", generator=g) < d[:, None])
+    start = torch.randint(0, cols - gap, (rows, 1), device="cuda", generator=g)
+    col = torch.arange(cols, device="cuda")[None, :]
+    W = W * ~((col >= start) & (col < start + gap))
+    W[::zero_every] = 0
+    x = torch.randn((cols,), device="cuda", dtype=torch.float32, generator=g).to(torch.float16)
+    return W.contiguous(), x
+
+
+def make_inputs(torch, suite):
+    """List of (rows, cols, label, W, x) for a workload."""
+    out = []
+    if suite == "llama":
+        for si, (rows, cols) in enumerate(SHAPES):
+            for di, d in enumerate(DENSITIES):
+                out.append((rows, cols, d, *make_pruned(torch, rows, cols, d, seed=1000 * si + di)))
+    elif suite == "large":
+        for si, (rows, cols) in enumerate(LARGE_SHAPES):
+            for di, d in enumerate(LARGE_DENSITIES):
+                out.append((rows, cols, d, *make_bernoulli(torch, rows, cols, d, seed=5000 + 100 * si + di)))
+    elif suite == "skew":
+        out.append((14336, 4096, "skewed", *make_skewed(torch, 14336, 4096, seed=9000)))
+        out.append((14336, 4096, 0.3, *make_bernoulli(torch, 14336, 4096, 0.3, seed=9001)))
+    else:
+        raise ValueError(suite)
+    return out
 
 
 def clone_compressed(c):
@@ -132,6 +199,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
     ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
+    ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
+                    help="llama = the headline workload; large / skew = the other shape families")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="also launch calibration_copy_kernel on a 256 MiB buffer this many times "
+                         "(reference dispatches for scaling rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (rows would shard across GPUs, but no "
@@ -148,23 +220,39 @@ def main():
 
     # ---- inputs ---------------------------------------------------------------------------------
     cases = []
-    for si, (rows, cols) in enumerate(SHAPES):
-        for di, d in enumerate(DENSITIES):
-            W, x = make_pruned(torch, rows, cols, d, seed=1000 * si + di)
-            c = mk.compress(W)
-            P = c[0].numel()
-            cases.append({"rows": rows, "cols": cols, "density": d, "P": P, "x": x,
-                          "copies": [c, clone_compressed(c)], "W": W,
-                          "bytes": algorithmic_bytes(P, rows, cols)})
-            log(f"case {rows}x{cols} d={d}: P={P} bytes={cases[-1]['bytes'] / 1e6:.1f} MB")
+    for rows, cols, d, W, x in make_inputs(torch, args.suite):
+        c = mk.compress(W)
+        P = c[0].numel()
+        cases.append({"rows": rows, "cols": cols, "density": d, "P": P, "x": x,
+                      "copies": [c, clone_compressed(c)], "W": W,
+                      "bytes": algorithmic_bytes(P, rows, cols)})
+        log(f"case {rows}x{cols} d={d}: P={P} bytes={cases[-1]['bytes'] / 1e6:.1f} MB")
     step_bytes = sum(c["bytes"] for c in cases)
     n_launch = len(cases)
 
     # correctness of what is about to be timed (cheap: one case per shape, fp32 dense product)
-    for c in cases[3::6]:
+    for c in cases[3::6] if args.suite == "llama" else cases:
         y = mk.multiply(c["copies"][0], c["x"]).float()
         want = c["W"].float() @ c["x"].float()
         assert torch.allclose(y, want, rtol=1e-2, atol=1e-3), "multiply disagrees with the dense product"
+
+    if args.calibration_copies > 0:
+        import ctypes
+
+        lib = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
+        lib.macko_calibration_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        n_bytes = 256 << 20
+        src = torch.ones(n_bytes // 2, dtype=torch.float16, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            rc = lib.macko_calibration_copy(src.data_ptr(), dst.data_ptr(), n_bytes,
+                                            torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        log(f"calibration: {args.calibration_copies} copies of {n_bytes} bytes "
+            f"(each reads {n_bytes} and writes {n_bytes} bytes)")
+        del src, dst
 
     # ---- the timed region: K steps replayed from graphs on a side stream --------------------------
     def step(copy):
@@ -238,7 +326,9 @@ def main():
     # ---- CPU baseline on a bounded sample --------------------------------------------------------
     cpu = None
     if not args.no_cpu_baseline:
-        sample = [(c["W"], c["x"], c["density"]) for c in cases if c["density"] == 0.5]
+        sample = [(c["W"], c["x"], c["density"]) for c in cases if c["density"] == 0.5 and c["rows"] * c["cols"] < 5e7]
+        if not sample:
+            sample = [(W, x, d) for _, _, d, W, x in make_inputs(torch, "llama") if d == 0.5]
         cpu = cpu_baseline(torch, sample)
         log("cpu baseline:", cpu)
 
@@ -261,9 +351,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": "configs[1]: Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as fp16 SpMV, "
-                        "per-row magnitude pruning, density in {0.1,0.2,0.3,0.5,0.7,0.9}; one step = one "
-                        "multiply of each of the 18 (shape, density) pairs, replayed from a HIP graph",
+            "workload": WORKLOADS[args.suite],
             "launches_per_step": n_launch,
             "bytes_per_step": step_bytes,
         },
@@ -275,8 +363,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBPS, 4),
-            "traffic": None,
-            "kernel": "spmv_rows_kernel",
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.suite),
+            "kernel": "spmv_stream_kernel",
             "bytes_per_launch": round(bytes_per_launch),
             "us_per_launch": round(launch_us, 3),
         },

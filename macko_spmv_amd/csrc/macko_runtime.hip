@@ -36,6 +36,26 @@ int device_info(DeviceInfo *out)
 
 }  // namespace macko
 
+// Plain 16-byte-per-thread copy with a recognisable name: hardware byte counters (FETCH_SIZE,
+// WRITE_SIZE) are scaled by what they report for this kernel on a buffer of known size.
+__global__ void __launch_bounds__(256) calibration_copy_kernel(const macko::u32x4 *__restrict__ src,
+                                                               macko::u32x4 *__restrict__ dst, size_t n_vec)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) dst[i] = src[i];
+}
+
+// Copies `bytes` (a multiple of 16; both pointers 16-byte aligned) from src to dst on `stream`.
+// Not part of the public ABI; used by the benchmark's counter calibration.
+extern "C" int macko_calibration_copy(const void *src, void *dst, int64_t bytes, void *stream)
+{
+    if (src == nullptr || dst == nullptr || bytes < 0 || (bytes & 15)) return MACKO_E_INVALID_ARGUMENT;
+    if (bytes == 0) return 0;
+    hipLaunchKernelGGL(calibration_copy_kernel, dim3(4096), dim3(256), 0, macko::as_stream(stream),
+                       (const macko::u32x4 *)src, (macko::u32x4 *)dst, (size_t)bytes / 16);
+    return (int)hipGetLastError();
+}
+
 extern "C" int macko_hip_abi_version(void) { return 1; }
 
 extern "C" const char *macko_hip_error_string(int code)
