@@ -465,69 +465,99 @@ spmv_stream_kernel(const SpmvArgs a)
     const u32 last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
 
     float acc0 = 0.f, acc1 = 0.f;
-    int carry = 0;  // nibble sum of the current row so far
     typedef __attribute__((address_space(3))) const uint16_t *lds_u16_ptr;
-    const u32 lds_base = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+    // LDS byte address of x[0] (x sits kLdsFront bytes into this kernel's dynamic LDS)
+    const u32 x_addr = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
+    // row_addr: LDS byte address the next entry of the current row would read if its nibble were 0,
+    // i.e. x_addr + 2 * (entries of the row consumed so far + their nibble sum).  Wave-uniform.
+    u32 row_addr = x_addr;
     MACKO_STAMP(5);
 
-    // One segment pass: entries [pos, seg_end) of tile `tb`, all in row r.
-    auto tile_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end) {
+    // The eight multiply-adds of a lane: entry k reads x at base + 2k + 2 * (nibbles 0..k), which is
+    // one v_dot8_u32_u4 with the multiplier 2 in the first k+1 nibble positions.
+    auto lane_fma = [&](const u32x4 &vv, u32 dd, u32 base) {
+        const u32 m[8] = {0x2u, 0x22u, 0x222u, 0x2222u, 0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const u32 addr = __builtin_amdgcn_udot8(dd, m[k], base, false);
+            uint16_t xb;
+#if defined(MACKO_EXP_NO_GATHER)
+            xb = (uint16_t)(addr & 0x3fffu);
+#else
+            if (X_LDS) {
+                xb = *reinterpret_cast<lds_u16_ptr>((u32)(addr + 2 * k));  // ds_read_u16 with offset 2k
+            } else {
+                int o = (int)(addr - x_addr) + 2 * k;
+                const int omax = 2 * a.cols - 2;
+                o = o < 0 ? 0 : (o > omax ? omax : o);
+                xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
+            }
+#endif
+            const u32 w = vv[k >> 1];
+            const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+            if (k & 1)
+                acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
+            else
+                acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
+        }
+    };
+
+    // A tile that lies wholly inside the current row: no masks, every lane active.  Each lane
+    // advances the row address by 16 bytes (its 8 entries) plus twice its nibble sum; the DPP scan
+    // of that quantity gives every lane its starting address.
+    auto full_tile_pass = [&](const u32x4 &vj, u32 dj) {
+#if defined(MACKO_EXP_NO_COMPUTE)
+        acc0 += __builtin_bit_cast(float, (vj.x ^ vj.y ^ vj.z ^ vj.w ^ dj) & 0x3fffffffu);
+        return;
+#endif
+        const u32 step = __builtin_amdgcn_udot8(dj, 0x22222222u, 16u, false);
+        const u32 incl = (u32)wave_scan_inclusive((int)step);
+        const u32 base = (incl - step) + row_addr;
+        row_addr += (u32)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        lane_fma(vj, dj, base);
+    };
+
+    // Entries [pos, seg_end) of the tile starting at entry `tb`, all in the current row: lanes
+    // outside the segment are switched off, the first and last lane of the segment are masked.
+    // A row that starts `q0` entries into its first lane shifts every address by -2*q0.
+    auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end) {
 #if defined(MACKO_EXP_NO_COMPUTE)
         acc0 += __builtin_bit_cast(float, (vj.x ^ vj.y ^ vj.z ^ vj.w ^ dj) & 0x3fffffffu);
         return;
 #endif
         const int rel0 = pos - tb;
         const int rel1 = seg_end - tb;
+        const int l0 = rel0 >> 3, q0 = rel0 & 7;
+        const int l1 = (rel1 - 1) >> 3, q1 = rel1 & 7;
         u32x4 vv = vj;
         u32 dd = dj;
-        bool active = true;
-        if (rel0 != 0 || rel1 != kTile) {  // not the whole tile (wave-uniform test)
-            const int l0 = rel0 >> 3, q0 = rel0 & 7;
-            const int l1 = (rel1 - 1) >> 3, q1 = rel1 & 7;
-            active = lane >= l0 && lane <= l1;
-            if (!active) dd = 0;
-            if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
-            if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
-        }
-        const int s = (int)__builtin_amdgcn_udot8(dd, 0x11111111u, 0u, false);
-        const int incl = wave_scan_inclusive(s);
-        // LDS byte address of x[col] for entry 0 of this chunk, before its own nibble:
-        // kLdsFront + 2 * (entry index in the row + nibbles before it); tb + 8*lane - e0 >= -7 for an
-        // active lane, so it stays positive.  The wave-uniform part is folded on the scalar unit.
-        const u32 uniform_part = lds_base + (u32)(kLdsFront + 2 * (tb - e0 + carry));
-        const u32 addr0 = ((u32)(incl - s) << 1) + (lane16 + uniform_part);
-        carry += __builtin_amdgcn_readlane(incl, kWave - 1);
-        if (active) {
-            const u32 m[8] = {0x2u, 0x22u, 0x222u, 0x2222u, 0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const u32 addr = __builtin_amdgcn_udot8(dd, m[k], addr0, false);
-                uint16_t xb;
-#if defined(MACKO_EXP_NO_GATHER)
-                xb = (uint16_t)(addr & 0x3fffu);
-#else
-                if (X_LDS) {
-                    // addr already carries the LDS base, so this is a bare ds_read_u16 with an
-                    // immediate offset
-                    xb = *reinterpret_cast<lds_u16_ptr>((u32)(addr + 2 * k));
-                } else {
-                    int o = (int)addr + 2 * k - kLdsFront;
-                    const int omax = 2 * a.cols - 2;
-                    o = o < 0 ? 0 : (o > omax ? omax : o);
-                    xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
-                }
-#endif
-                const u32 w = vv[k >> 1];
-                const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
-                if (k & 1)
-                    acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
-                else
-                    acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
-            }
-        }
+        const bool active = lane >= l0 && lane <= l1;
+        if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
+        if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
+        u32 step = __builtin_amdgcn_udot8(dd, 0x22222222u, 16u, false);
+        step = active ? step : 0u;
+        const u32 incl = (u32)wave_scan_inclusive((int)step);
+        const u32 origin = row_addr - 2u * (u32)q0;
+        const u32 base = (incl - step) + origin;
+        row_addr = origin + (u32)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        if (active) lane_fma(vv, dd, base);
     };
 
-    // Fill the ring with my first D tiles, then: take a slot, process it, refill it.  Every step
+    auto finish_row = [&]() {
+        store_row(r, wave_sum(acc0 + acc1));
+        acc0 = acc1 = 0.f;
+        row_addr = x_addr;
+        do {  // next non-empty owned row; empty ones get their zero on the way
+            ++r;
+            if (r >= row_last) break;  // then the row just finished ended at s_end and all loops end
+            slide_window(r);
+            e0 = row_start(r);
+            e1 = row_start(r + 1);
+            if (e1 == e0) store_row(r, 0.f);
+        } while (e1 == e0);
+    };
+
+    // Fill the ring with my first D tiles, then: take a slot, refill it, process.  Every step
     // issues exactly two loads (a "no tile" address once the range is exhausted), so a slot's
     // loads are always followed by those of the D - 1 other slots when it is awaited.
     static_for<D>([&](auto slot) {
@@ -544,25 +574,20 @@ spmv_stream_kernel(const SpmvArgs a)
             ring_take<D, J, kTileLoads - 2>(vj, dj);
             issue_slot(slot, tile + D, tile + D < last_tile);  // refill at once: the copy is out
             const int tb = (int)(tile << kTileShift);
-            const int lim = tb + kTile < s_end ? tb + kTile : s_end;
-            int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
-            while (pos < lim) {
-                const int seg_end = e1 < lim ? e1 : lim;
-                tile_pass(vj, dj, tb, pos, seg_end);
-                if (seg_end == e1) {  // row finished
-                    store_row(r, wave_sum(acc0 + acc1));
-                    acc0 = acc1 = 0.f;
-                    carry = 0;
-                    do {  // next non-empty owned row; empty ones get their zero on the way
-                        ++r;
-                        if (r >= row_last) break;  // then seg_end == s_end == lim and all loops end
-                        slide_window(r);
-                        e0 = row_start(r);
-                        e1 = row_start(r + 1);
-                        if (e1 == e0) store_row(r, 0.f);
-                    } while (e1 == e0);
+            const int tile_end = tb + kTile;
+            if (e0 <= tb && e1 >= tile_end) {  // the common case for rows longer than a tile
+                full_tile_pass(vj, dj);
+                if (e1 == tile_end) finish_row();
+            } else {
+                const int lim = tile_end < s_end ? tile_end : s_end;
+                int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
+                while (pos < lim) {
+                    const int seg_end = e1 < lim ? e1 : lim;
+                    segment_pass(vj, dj, tb, pos, seg_end);
+                    const bool row_done = seg_end == e1;
+                    pos = seg_end;
+                    if (row_done) finish_row();
                 }
-                pos = seg_end;
             }
         });
     }
