@@ -253,7 +253,10 @@ template <int D, int J>
 __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
                                            const u32x4 &buf_deltas)
 {
-    static_assert(D == 4 || D == 8 || D == 16, "ring depth");
+    static_assert(D == 1 || D == 2 || D == 4 || D == 8 || D == 16, "ring depth");
+    if (D == 1 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v92", MACKO_FIXED_CLOBBERS_4);
+    if (D == 2 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v96", MACKO_FIXED_CLOBBERS_4);
+    if (D == 2 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v97", MACKO_FIXED_CLOBBERS_4);
     if (D == 4 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v104", MACKO_FIXED_CLOBBERS_4);
     if (D == 4 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v105", MACKO_FIXED_CLOBBERS_4);
     if (D == 4 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v106", MACKO_FIXED_CLOBBERS_4);
@@ -287,6 +290,9 @@ __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset,
 template <int D, int J, int N>
 __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
 {
+    if (D == 1 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v92");
+    if (D == 2 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v96");
+    if (D == 2 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v97");
     if (D == 4 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v104");
     if (D == 4 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v105");
     if (D == 4 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v106");
@@ -631,7 +637,7 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 // Launch-shape overrides for tuning runs (0 = built-in default).  Not part of the public ABI.
 struct Tuning {
     int block;      // threads per workgroup: 256, 512 or 1024
-    int depth;      // tiles in flight per wave: 4, 8 or 16 (16 only with 256 or 512 threads)
+    int depth;      // tiles in flight per wave: 1, 2, 4 or 8 (not every block size has every depth)
     int wg_per_cu;  // workgroups launched per compute unit
 };
 Tuning g_tuning = {0, 0, 0};
@@ -651,7 +657,7 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 
     const Tuning t = g_tuning;
     const int block = t.block ? t.block : 1024;
-    const int depth = t.depth ? t.depth : 4;
+    const int depth = t.depth ? t.depth : 2;
     const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
     const int waves = block / kWave;
     // at most one wave per tile: tiny matrices get a small grid
@@ -661,18 +667,18 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     if (grid < 1) grid = 1;
 
     const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
-    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 4, false, AXPBY>(a, (int)grid, 0, stream);
+    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 2, false, AXPBY>(a, (int)grid, 0, stream);
 #define MACKO_CASE(B, D_) \
     if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
-    MACKO_CASE(1024, 4)
+    MACKO_CASE(1024, 2)
     if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
+        MACKO_CASE(1024, 1)
+        MACKO_CASE(1024, 4)
         MACKO_CASE(1024, 8)
+        MACKO_CASE(512, 2)
         MACKO_CASE(512, 4)
-        MACKO_CASE(512, 8)
-        MACKO_CASE(512, 16)
+        MACKO_CASE(256, 2)
         MACKO_CASE(256, 4)
-        MACKO_CASE(256, 8)
-        MACKO_CASE(256, 16)
     }
 #undef MACKO_CASE
     return MACKO_E_INVALID_ARGUMENT;
