@@ -414,33 +414,15 @@ spmv_stream_kernel(const SpmvArgs a)
     const int row_last = uniform(range[1]);
     MACKO_STAMP(2);
 
-    // ---- 4. x pieces into LDS ---------------------------------------------------------------------------
-    if (X_LDS) {
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(lds + kLdsFront);
-        const u32x4 x0 = xpiece_take<0, 1>();
-        if (tid < x_nvec) d4[tid] = x0;
-        const u32x4 x1 = xpiece_take<1, 0>();
-        if (tid + BLOCK < x_nvec) d4[tid + BLOCK] = x1;
-        MACKO_STAMP(3);
-        __syncthreads();
-    }
-    MACKO_STAMP(4);
-
-    if (row_first >= row_last) return;
-
-    // ---- 6. stream ----------------------------------------------------------------------------------
+    // ---- 4. my first row and my tile range --------------------------------------------------------------
     // window of row_ptr values: lane i holds row_ptr[win_base + i]
     int win_base = base[0];
     int win = window[0];
-    if (row_first < win_base || row_first + 1 > win_base + 63) {
-        win_base = row_first;
-        win = load_row_window(a.row_ptr, a.rows, win_base, lane);
-    }
     auto row_start = [&](int r) -> int {  // r in [win_base, win_base + 63]
         return __builtin_amdgcn_readlane(win, r - win_base);
     };
     auto slide_window = [&](int r) {  // make rows r and r + 1 addressable
-        if (r + 1 > win_base + 63) {
+        if (r < win_base || r + 1 > win_base + 63) {
             win_base = r;
             win = load_row_window(a.row_ptr, a.rows, win_base, lane);
         }
@@ -454,22 +436,60 @@ spmv_stream_kernel(const SpmvArgs a)
     };
 
     // current row r = first non-empty owned row; empty ones are written on the way
+    bool have_work = row_first < row_last;
     int r = row_first;
-    int e0 = row_start(r);
-    int e1 = row_start(r + 1);
-    while (e1 == e0) {
-        store_row(r, 0.f);
-        ++r;
-        if (r >= row_last) return;
+    int e0 = 0, e1 = 0, s_end = 0;
+    u32 first_tile = 0, last_tile = 0;
+    if (have_work) {
         slide_window(r);
         e0 = row_start(r);
         e1 = row_start(r + 1);
+        while (e1 == e0) {
+            store_row(r, 0.f);
+            ++r;
+            if (r >= row_last) {
+                have_work = false;
+                break;
+            }
+            slide_window(r);
+            e0 = row_start(r);
+            e1 = row_start(r + 1);
+        }
     }
-    // end of my last owned row
-    const int s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
-    const u32 first_tile = (u32)e0 >> kTileShift;
-    const u32 last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
+    if (have_work) {
+        // end of my last owned row
+        s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
+        first_tile = (u32)e0 >> kTileShift;
+        last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
+        // Fill the ring with my first D tiles before x is even in LDS: they fly while the
+        // workgroup finishes the copy and meets at the barrier.
+        static_for<D>([&](auto slot) {
+            constexpr int J = decltype(slot)::value;
+            issue_slot(slot, first_tile + J, first_tile + J < last_tile);
+        });
+    }
 
+    // ---- 5. x pieces into LDS (older than the ring loads just issued, if any) ---------------------------
+    if (X_LDS) {
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(lds + kLdsFront);
+        u32x4 x0, x1;
+        if (have_work) {
+            x0 = xpiece_take<0, kTileLoads + 1>();
+            x1 = xpiece_take<1, kTileLoads>();
+        } else {
+            x0 = xpiece_take<0, 1>();
+            x1 = xpiece_take<1, 0>();
+        }
+        if (tid < x_nvec) d4[tid] = x0;
+        if (tid + BLOCK < x_nvec) d4[tid + BLOCK] = x1;
+        MACKO_STAMP(3);
+        __syncthreads();
+    }
+    MACKO_STAMP(4);
+
+    if (!have_work) return;
+
+    // ---- 6. stream ----------------------------------------------------------------------------------
     float acc0 = 0.f, acc1 = 0.f;
     typedef __attribute__((address_space(3))) const uint16_t *lds_u16_ptr;
     // LDS byte address of x[0] (x sits kLdsFront bytes into this kernel's dynamic LDS)
@@ -563,13 +583,9 @@ spmv_stream_kernel(const SpmvArgs a)
         } while (e1 == e0);
     };
 
-    // Fill the ring with my first D tiles, then: take a slot, refill it, process.  Every step
-    // issues exactly two loads (a "no tile" address once the range is exhausted), so a slot's
-    // loads are always followed by those of the D - 1 other slots when it is awaited.
-    static_for<D>([&](auto slot) {
-        constexpr int J = decltype(slot)::value;
-        issue_slot(slot, first_tile + J, first_tile + J < last_tile);
-    });
+    // The ring holds my first D tiles; now: take a slot, refill it, process.  Every step issues
+    // exactly two loads (a "no tile" address once the range is exhausted), so a slot's loads are
+    // always followed by those of the D - 1 other slots when it is awaited.
     for (u32 tile0 = first_tile; tile0 < last_tile; tile0 += D) {
         static_for<D>([&](auto slot) {
             constexpr int J = decltype(slot)::value;
@@ -660,9 +676,13 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     const int depth = t.depth ? t.depth : 2;
     const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
     const int waves = block / kWave;
-    // at most one wave per tile: tiny matrices get a small grid
+    // about one wave per tile at most, so tiny matrices get a small grid; but when rows are about
+    // a tile long, prefer one wave per row over a slightly smaller wave count that would leave
+    // some waves with two rows
     const long long n_tiles = (a.padded + kTile - 1) / kTile;
-    long long grid = (n_tiles + waves - 1) / waves;
+    long long waves_wanted = n_tiles;
+    if (a.rows > waves_wanted) waves_wanted = a.rows < 2 * n_tiles ? a.rows : 2 * n_tiles;
+    long long grid = (waves_wanted + waves - 1) / waves;
     if (grid > (long long)info.compute_units * wg_per_cu) grid = (long long)info.compute_units * wg_per_cu;
     if (grid < 1) grid = 1;
 
