@@ -1,0 +1,320 @@
+"""Llama-architecture batch-1 decode with MACKO linear layers.
+
+Counterpart of the upstream helper scripts:
+  python_scripts/util_compress_llm.py:16-44    -> compress_state_dict()  (keys `<module>.c_0 .. c_4`)
+  python_scripts/util_run_pruned_llm.py:102-133 -> MackoLinear (their CustomLayer), load_compressed_linears (their fix)
+  python_scripts/util_run_pruned_llm.py:51-99,136-207 -> Generator-style greedy decode loop and the tok/s, memory report
+
+The upstream scripts wrap a Hugging Face checkpoint and tokenizer fetched by name; neither exists
+offline, so the model here is a self-contained decoder with the same architecture and the same
+parameter names (`model.layers.{i}.self_attn.q_proj.weight`, ...), randomly initialised, and the
+prompt is random token ids.  Decode steps are captured in a HIP graph (the upstream script uses
+torch.compile(mode="reduce-overhead") for the same purpose).
+
+Run:  python -m macko_spmv_amd.llm --density 0.5            (prints one JSON line)
+"""
+import argparse
+import json
+import math
+import sys
+import time
+from collections import OrderedDict
+
+import torch
+from torch import nn
+
+import macko_spmv_amd as macko_spmv
+
+PROJECTIONS = (("self_attn", "q_proj"), ("self_attn", "k_proj"), ("self_attn", "v_proj"), ("self_attn", "o_proj"),
+               ("mlp", "gate_proj"), ("mlp", "up_proj"), ("mlp", "down_proj"))
+
+
+def is_compressible(key):
+    """Same rule as upstream compress_k: attention and MLP weight matrices only."""
+    return ("weight" in key) and ("self_attn" in key or "mlp" in key)
+
+
+def compress_state_dict(state_dict, compress=None):
+    """state_dict -> OrderedDict where every compressible `<m>.weight` became `<m>.c_0 .. <m>.c_4`
+    (values, deltas, row_indices, rows, cols); other entries pass through.  Keys are visited in
+    sorted order like upstream."""
+    compress = compress or macko_spmv.compress
+    out = OrderedDict()
+    for key in sorted(state_dict.keys()):
+        value = state_dict[key]
+        if is_compressible(key):
+            compressed = compress(value.contiguous())
+            for i in range(5):
+                out[key.replace("weight", f"c_{i}")] = compressed[i]
+        else:
+            out[key] = value
+    return out
+
+
+class MackoLinear(nn.Module):
+    """y = M x for a compressed M; x of shape (..., cols) -> (..., rows)."""
+
+    def __init__(self, c_0, c_1, c_2, c_3, c_4):
+        super().__init__()
+        self.register_buffer("c_0", c_0)
+        self.register_buffer("c_1", c_1)
+        self.register_buffer("c_2", c_2)
+        self.c_3 = int(c_3)
+        self.c_4 = int(c_4)
+
+    def forward(self, x):
+        lead = x.shape[:-1]
+        flat = x.reshape(-1, self.c_4)
+        compressed = (self.c_0, self.c_1, self.c_2, self.c_3, self.c_4)
+        if flat.shape[0] == 1:
+            out = macko_spmv.multiply(compressed, flat[0].contiguous()).unsqueeze(0)
+        else:  # one product per row of x, as the upstream vmap fallback does
+            out = torch.stack([macko_spmv.multiply(compressed, row.contiguous()) for row in flat])
+        return out.reshape(*lead, self.c_3)
+
+    def weight_bytes(self):
+        return self.c_0.numel() * 2 + self.c_1.numel() + self.c_2.numel() * 4
+
+
+def load_compressed_linears(model, compressed_sd):
+    """Swap the seven projections of every layer for MackoLinear built from `compressed_sd`."""
+    for i, layer in enumerate(model.model.layers):
+        for parent, name in PROJECTIONS:
+            path = f"model.layers.{i}.{parent}.{name}"
+            setattr(getattr(layer, parent), name,
+                    MackoLinear(*[compressed_sd[f"{path}.c_{k}"] for k in range(5)]))
+    return model
+
+
+# ---- a minimal Llama-architecture decoder (batch 1) ------------------------------------------------
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim, eps=1e-5):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        v = x.float()
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.eps)
+        return (v * self.weight.float()).to(x.dtype)
+
+
+class Attention(nn.Module):
+    def __init__(self, dim, n_heads, max_len):
+        super().__init__()
+        self.n_heads, self.head_dim, self.max_len = n_heads, dim // n_heads, max_len
+        self.q_proj = nn.Linear(dim, dim, bias=False)
+        self.k_proj = nn.Linear(dim, dim, bias=False)
+        self.v_proj = nn.Linear(dim, dim, bias=False)
+        self.o_proj = nn.Linear(dim, dim, bias=False)
+        self.register_buffer("k_cache", torch.zeros(1, n_heads, max_len, self.head_dim), persistent=False)
+        self.register_buffer("v_cache", torch.zeros(1, n_heads, max_len, self.head_dim), persistent=False)
+
+    def forward(self, x, cos, sin, positions, mask):
+        t = x.shape[1]
+        q = self.q_proj(x).view(1, t, self.n_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(x).view(1, t, self.n_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(x).view(1, t, self.n_heads, self.head_dim).transpose(1, 2)
+        q, k = _rope(q, cos, sin), _rope(k, cos, sin)
+        self.k_cache.index_copy_(2, positions, k)
+        self.v_cache.index_copy_(2, positions, v)
+        att = torch.matmul(q, self.k_cache.transpose(2, 3)) / math.sqrt(self.head_dim)
+        att = torch.softmax((att + mask).float(), dim=-1).to(x.dtype)
+        out = torch.matmul(att, self.v_cache).transpose(1, 2).reshape(1, t, -1)
+        return self.o_proj(out)
+
+
+def _rope(x, cos, sin):
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
+    return x * cos + torch.cat((-x2, x1), dim=-1) * sin
+
+
+class MLP(nn.Module):
+    def __init__(self, dim, hidden):
+        super().__init__()
+        self.gate_proj = nn.Linear(dim, hidden, bias=False)
+        self.up_proj = nn.Linear(dim, hidden, bias=False)
+        self.down_proj = nn.Linear(hidden, dim, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class Block(nn.Module):
+    def __init__(self, dim, hidden, n_heads, max_len):
+        super().__init__()
+        self.self_attn = Attention(dim, n_heads, max_len)
+        self.mlp = MLP(dim, hidden)
+        self.input_layernorm = RMSNorm(dim)
+        self.post_attention_layernorm = RMSNorm(dim)
+
+    def forward(self, x, cos, sin, positions, mask):
+        x = x + self.self_attn(self.input_layernorm(x), cos, sin, positions, mask)
+        return x + self.mlp(self.post_attention_layernorm(x))
+
+
+class _Body(nn.Module):
+    def __init__(self, vocab, dim, hidden, n_layers, n_heads, max_len):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(vocab, dim)
+        self.layers = nn.ModuleList([Block(dim, hidden, n_heads, max_len) for _ in range(n_layers)])
+        self.norm = RMSNorm(dim)
+
+
+class LlamaDecoder(nn.Module):
+    """Parameter names follow the Hugging Face Llama layout so compressed state dicts are
+    interchangeable with the upstream scripts' (`model.layers.{i}.mlp.up_proj.c_0`, ...)."""
+
+    def __init__(self, vocab=32000, dim=4096, hidden=11008, n_layers=32, n_heads=32, max_len=512):
+        super().__init__()
+        self.max_len, self.head_dim = max_len, dim // n_heads
+        self.model = _Body(vocab, dim, hidden, n_layers, n_heads, max_len)
+        self.lm_head = nn.Linear(dim, vocab, bias=False)
+        inv = 1.0 / (10000.0 ** (torch.arange(0, self.head_dim, 2).float() / self.head_dim))
+        ang = torch.outer(torch.arange(max_len).float(), inv)
+        ang = torch.cat((ang, ang), dim=-1)
+        self.register_buffer("cos", ang.cos(), persistent=False)
+        self.register_buffer("sin", ang.sin(), persistent=False)
+
+    def forward(self, tokens, positions):
+        """tokens (1, t) int64, positions (t,) int64 -> logits (1, t, vocab)."""
+        x = self.model.embed_tokens(tokens)
+        cos = self.cos[positions].to(x.dtype)[None, None]
+        sin = self.sin[positions].to(x.dtype)[None, None]
+        key_pos = torch.arange(self.max_len, device=tokens.device)
+        mask = torch.where(key_pos[None, :] <= positions[:, None], 0.0, float("-inf")).to(x.dtype)[None, None]
+        for layer in self.model.layers:
+            x = layer(x, cos, sin, positions, mask)
+        return self.lm_head(self.model.norm(x))
+
+
+def prune_rows_(weight, density):
+    """In place: keep the round(density * cols) largest |w| of every row."""
+    keep = int(round(density * weight.shape[1]))
+    if keep < weight.shape[1]:
+        idx = weight.abs().float().topk(keep, dim=1).indices
+        mask = torch.zeros_like(weight, dtype=torch.bool)
+        mask.scatter_(1, idx, True)
+        weight.mul_(mask)
+    return weight
+
+
+@torch.no_grad()
+def greedy_decode(model, prompt, new_tokens, use_graph=True):
+    """Prefill `prompt` (1, t), then generate `new_tokens` greedily, one token per step.
+    Returns (generated ids (new_tokens,), seconds spent in the decode steps)."""
+    device = prompt.device
+    t = prompt.shape[1]
+    logits = model(prompt, torch.arange(t, device=device))
+    token = logits[:, -1].argmax(-1, keepdim=True)           # (1, 1)
+    position = torch.tensor([t], device=device)
+    out = torch.zeros(new_tokens, dtype=torch.long, device=device)
+    out[0] = token[0, 0]
+
+    def step():
+        nxt = model(token, position)[:, -1].argmax(-1, keepdim=True)
+        token.copy_(nxt)
+        position.add_(1)
+
+    graph = None
+    if use_graph:
+        state = (token.clone(), position.clone())
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()                                            # warm-up outside capture
+            side.synchronize()
+            token.copy_(state[0])
+            position.copy_(state[1])
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                step()
+            token.copy_(state[0])
+            position.copy_(state[1])
+        torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for i in range(1, new_tokens):
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+        out[i] = token[0, 0]
+    torch.cuda.synchronize()
+    return out, time.perf_counter() - start
+
+
+def build_model(density, n_layers, dim, hidden, n_heads, vocab, max_len, seed=0, sparse=True):
+    """Random Llama-architecture fp16 model on the GPU with every projection pruned per row to
+    `density`; with sparse=True the projections are replaced by MackoLinear.  Returns (model, bytes
+    held by the projection weights)."""
+    torch.manual_seed(seed)
+    model = LlamaDecoder(vocab, dim, hidden, n_layers, n_heads, max_len).half().cuda()
+    proj_bytes = 0
+    for i, layer in enumerate(model.model.layers):
+        for parent, name in PROJECTIONS:
+            lin = getattr(getattr(layer, parent), name)
+            w = lin.weight.data
+            w.normal_(0.0, 0.02)
+            if density < 1.0:
+                prune_rows_(w, density)
+            if sparse:
+                new = MackoLinear(*macko_spmv.compress(w.contiguous()))
+                setattr(getattr(layer, parent), name, new)
+                proj_bytes += new.weight_bytes()
+            else:
+                proj_bytes += w.numel() * 2
+    torch.cuda.empty_cache()
+    return model, proj_bytes
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="batch-1 greedy decode, dense vs MACKO projections")
+    ap.add_argument("--density", type=float, default=0.5)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--dim", type=int, default=4096)
+    ap.add_argument("--hidden", type=int, default=11008)
+    ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--vocab", type=int, default=32000)
+    ap.add_argument("--prompt", type=int, default=128)
+    ap.add_argument("--tokens", type=int, default=256)
+    ap.add_argument("--runs", type=int, default=3)
+    ap.add_argument("--skip-dense", action="store_true")
+    args = ap.parse_args(argv)
+    assert torch.cuda.is_available(), "needs a GPU"
+    torch.set_grad_enabled(False)
+    max_len = args.prompt + args.tokens + 8
+    result = {"density": args.density, "layers": args.layers, "prompt": args.prompt, "tokens": args.tokens}
+    for label, sparse in (("dense", False), ("macko", True)):
+        if label == "dense" and args.skip_dense:
+            continue
+        model, proj_bytes = build_model(args.density, args.layers, args.dim, args.hidden, args.heads, args.vocab,
+                                        max_len, sparse=sparse)
+        resident = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()  # the peak below covers prefill + decode, not model construction
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1)
+        prompt = torch.randint(0, args.vocab, (1, args.prompt), device="cuda", generator=g)
+        times = []
+        for _ in range(args.runs):
+            ids, seconds = greedy_decode(model, prompt, args.tokens)
+            times.append(seconds)
+        best = min(times)
+        result[label] = {
+            "tokens_per_s": round((args.tokens - 1) / best, 2),
+            "projection_weights_gb": round(proj_bytes / 1e9, 3),
+            "model_memory_gb": round(resident / 1e9, 3),
+            "peak_memory_gb": round(torch.cuda.max_memory_allocated() / 1e9, 3),
+            "first_tokens": ids[:8].tolist(),
+        }
+        print(label, result[label], file=sys.stderr, flush=True)
+        del model
+        torch.cuda.empty_cache()
+    if "dense" in result and "macko" in result:
+        result["speedup"] = round(result["macko"]["tokens_per_s"] / result["dense"]["tokens_per_s"], 3)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
