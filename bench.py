@@ -198,6 +198,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
+    ap.add_argument("--no-compress", action="store_true", help="skip the compressor timing")
     ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
     ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
                     help="llama = the headline workload; large / skew = the other shape families")
@@ -323,6 +324,30 @@ def main():
             })
             log(per_case[-1])
 
+    # ---- the compressor: whole compress() call (count pass, read-back of the total, fill pass) -----
+    compress_cases = []
+    if not args.no_compress:
+        for c in cases:
+            if c["density"] != 0.5:
+                continue
+            W = c["W"]
+            for _ in range(2):
+                comp = mk.compress(W)
+            torch.cuda.synchronize()
+            reps = 5
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                comp = mk.compress(W)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / reps
+            # both passes read the dense matrix; the second writes values, nibbles; row_ptr is written twice
+            nbytes = 2 * dense_bytes(c["rows"], c["cols"]) + 2.5 * comp[0].numel() + 8 * (c["rows"] + 1)
+            entry = {"shape": f"{c['rows']}x{c['cols']}", "density": c["density"], "us": round(dt * 1e6, 1),
+                     "gbps": round(nbytes / dt / 1e9, 1),
+                     "pct_hbm_peak": round(100 * nbytes / dt / 1e9 / HBM_PEAK_GBPS, 1)}
+            compress_cases.append(entry)
+            log("compress:", entry)
+
     # ---- CPU baseline on a bounded sample --------------------------------------------------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -370,6 +395,7 @@ def main():
         },
         "cpu_baseline": cpu,
         "cases": per_case,
+        "compress": compress_cases,
         "device": dev.name,
     }
     print(json.dumps(out), flush=True)

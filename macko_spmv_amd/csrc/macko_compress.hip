@@ -126,89 +126,147 @@ __global__ void __launch_bounds__(1024) scan_rows_kernel(int *__restrict__ row_p
     if (tid == 0) row_ptr[0] = 0;
 }
 
+// Packs the low nibbles of 8 staged entries (bits 16..19 of each word) into one delta word.
+__device__ __forceinline__ u32 pack_nibbles(const u32 (&e)[8])
+{
+    u32 w = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w |= ((e[i] >> 16) & 15u) << (4 * i);
+    return w;
+}
+
+// Orders this wave's LDS writes before its later LDS reads (the staging area is private to
+// the wave, so no workgroup barrier is involved).
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// Pass 2.  The wave stages the entries of its row in LDS at the offset they have inside their
+// 8-entry group of the output, so that every complete group leaves as one 16-byte store of
+// values and one 4-byte store of nibbles.  Groups cut by a row boundary are shared with the
+// neighbouring row's wave: their values go out as 2-byte stores and their nibbles are OR-ed
+// into the (zeroed) delta word.  `deltas` must be zero on entry; `values` need not be.
 __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__restrict__ dense, int rows,
                                                            int cols, const int *__restrict__ row_ptr,
                                                            uint16_t *__restrict__ values,
-                                                           unsigned char *__restrict__ deltas)
+                                                           u32 *__restrict__ delta_words, int padded)
 {
-    __shared__ uint16_t stage_values[kRowsPerBlock][kTile];
-    __shared__ unsigned char stage_nibbles[kRowsPerBlock][kTile];
+    constexpr int kStage = kTile + 8;  // a tile's entries plus the carried part of a group
+    __shared__ u32 stage_all[kRowsPerBlock][kStage];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
     const int row = blockIdx.x * kRowsPerBlock + wave;
-    const bool live = row < rows;
-    const int e0 = live ? row_ptr[row] : 0;
-    const int e1 = live ? row_ptr[row + 1] : 0;
-    const uint16_t *src = dense + (size_t)(live ? row : 0) * (size_t)cols;
-    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
-    uint16_t *sv = stage_values[wave];
-    unsigned char *sn = stage_nibbles[wave];
-    u32 *words = reinterpret_cast<u32 *>(deltas);
+    if (row >= rows) return;
+    const int e0 = row_ptr[row];
+    const int e1 = row_ptr[row + 1];
+    u32 *stage = stage_all[wave];
+    u32x4 *value_groups = reinterpret_cast<u32x4 *>(values);
 
+    if (row == rows - 1) {  // the unused tail of the last 8-entry group
+        for (int i = e1 + lane; i < padded; i += kWave) values[i] = 0;
+    }
+    if (e0 == e1) return;
+
+    const uint16_t *src = dense + (size_t)row * (size_t)cols;
+    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+
+    // stage[i] holds output entry base + i; [lo, hi) is staged and not yet written out
+    int base = e0 & ~7;
+    int lo = e0 - base;
+    int hi = lo;
     int carry = -1;
-    int pos = e0;  // next entry index to write
-    for (int c0 = 0; c0 < cols; c0 += kTile) {
-        int n_write = 0;
-        if (pos < e1) {  // wave-uniform
-            const int col = c0 + lane * kChunk;
-            const u32x4 v = load8(src, col, cols, vector_ok && col < cols);
-            const u32 nz = nonzero_bits(v);
-            const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
-            int pass_last;
-            int p = previous_nonzero(own_last, carry, lane, pass_last);
-            carry = pass_last > carry ? pass_last : carry;
-            // which of my 8 columns store an entry, and with which nibble
-            u32 entry_bits = 0;
-            u32 nibbles = 0;
+
+    // writes out groups [0, n_groups) of the stage; group g holds entries [a, b) with
+    // a = lo for group 0 and b = hi - 8g for a last, incomplete group
+    auto flush = [&](int n_groups) {
+        for (int g = lane; g < n_groups; g += kWave) {
+            u32 e[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int x = col + i;
-                const int dist = x - p;
-                const bool is_nz = (nz >> i) & 1u;
-                const bool is_entry = x < cols && (is_nz || (dist & 15) == 0);
-                const u32 nib = is_nz ? (u32)(dist - 1) & 15u : 15u;
-                entry_bits |= (is_entry ? 1u : 0u) << i;
-                nibbles |= nib << (4 * i);
-                p = is_nz ? x : p;
-            }
-            const int mine = __builtin_popcount(entry_bits);
-            const int incl = wave_scan_inclusive(mine);
-            const int produced = __builtin_amdgcn_readlane(incl, kWave - 1);
-            int slot = incl - mine;
+            for (int i = 0; i < 8; ++i) e[i] = stage[8 * g + i];
+            const int a = g == 0 ? lo : 0;
+            const int b = hi - 8 * g < 8 ? hi - 8 * g : 8;
+            const int out = (base >> 3) + g;
+            if (a == 0 && b == 8) {
+                u32x4 v;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if (entry_bits & (1u << i)) {
-                    u32 h = half_at(v, i);
-                    h = (h & 0x7fffu) > 0x7c00u ? 0x7fffu : h;
-                    sv[slot] = (uint16_t)h;
-                    sn[slot] = (unsigned char)((nibbles >> (4 * i)) & 15u);
-                    ++slot;
+                for (int i = 0; i < 4; ++i) v[i] = (e[2 * i] & 0xffffu) | (e[2 * i + 1] << 16);
+                value_groups[out] = v;
+                delta_words[out] = pack_nibbles(e);
+            } else {
+                u32 keep = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i >= a && i < b) {
+                        values[8 * (size_t)out + i] = (uint16_t)e[i];
+                        keep |= 15u << (4 * i);
+                    }
                 }
+                atomicOr(&delta_words[out], pack_nibbles(e) & keep);
             }
-            // entries past e1 are padding entries behind the row's last non-zero: not stored
-            n_write = produced < e1 - pos ? produced : e1 - pos;
         }
-        __syncthreads();  // staged entries visible to the whole wave
-        if (n_write > 0) {
-            for (int k = lane; k < n_write; k += kWave) values[pos + k] = sv[k];
-            // nibble pairs that live wholly inside [pos, pos + n_write) are plain byte stores;
-            // a lone nibble at either end shares its byte with a neighbour and is OR-ed in
-            const int first_even = pos + (pos & 1);
-            const int last_even = (pos + n_write) & ~1;
-            for (int e = first_even + 2 * lane; e < last_even; e += 2 * kWave)
-                deltas[e >> 1] = (unsigned char)(sn[e - pos] | (sn[e + 1 - pos] << 4));
-            if (lane == 0 && (pos & 1)) {
-                const int byte = pos >> 1;
-                atomicOr(&words[byte >> 2], ((u32)sn[0] << 4) << (8 * (byte & 3)));
-            }
-            if (lane == 1 && ((pos + n_write) & 1)) {
-                const int e = pos + n_write - 1;
-                const int byte = e >> 1;
-                atomicOr(&words[byte >> 2], (u32)sn[e - pos] << (8 * (byte & 3)));
-            }
-            pos += n_write;
+    };
+
+    u32x4 next = load8(src, lane * kChunk, cols, vector_ok && lane * kChunk < cols);
+    for (int c0 = 0; c0 < cols; c0 += kTile) {
+        const int col = c0 + lane * kChunk;
+        const u32x4 v = next;
+        if (c0 + kTile < cols) {
+            const int ncol = col + kTile;
+            next = load8(src, ncol, cols, vector_ok && ncol < cols);
         }
-        __syncthreads();  // staging buffers are reused by the next pass
+        const u32 nz = nonzero_bits(v);
+        const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
+        int pass_last;
+        int p = previous_nonzero(own_last, carry, lane, pass_last);
+        carry = pass_last > carry ? pass_last : carry;
+        // which of my 8 columns store an entry, and with which nibble
+        u32 entry_bits = 0;
+        u32 nibbles = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int x = col + i;
+            const int dist = x - p;
+            const bool is_nz = (nz >> i) & 1u;
+            const bool is_entry = x < cols && (is_nz || (dist & 15) == 0);
+            const u32 nib = is_nz ? (u32)(dist - 1) & 15u : 15u;
+            entry_bits |= (is_entry ? 1u : 0u) << i;
+            nibbles |= nib << (4 * i);
+            p = is_nz ? x : p;
+        }
+        const int mine = __builtin_popcount(entry_bits);
+        const int incl = wave_scan_inclusive(mine);
+        const int produced = __builtin_amdgcn_readlane(incl, kWave - 1);
+        // entries past e1 are padding entries behind the row's last non-zero: not stored
+        const int room = e1 - (base + hi);
+        const int n_new = produced < room ? produced : room;
+        int slot = incl - mine;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if ((entry_bits & (1u << i)) && slot < n_new) {
+                u32 h = half_at(v, i);
+                h = (h & 0x7fffu) > 0x7c00u ? 0x7fffu : h;
+                stage[hi + slot] = h | (((nibbles >> (4 * i)) & 15u) << 16);
+                ++slot;
+            }
+        }
+        hi += n_new;
+        wave_lds_fence();
+        const bool row_done = base + hi == e1;
+        const int n_groups = row_done ? (hi + 7) >> 3 : hi >> 3;
+        flush(n_groups);
+        if (row_done) break;
+        if (n_groups > 0) {  // carry the incomplete group to the front of the stage
+            const int rest = hi & 7;
+            const u32 moved = lane < rest ? stage[8 * n_groups + lane] : 0u;
+            wave_lds_fence();
+            if (lane < rest) stage[lane] = moved;
+            base += 8 * n_groups;
+            lo = 0;
+            hi = rest;
+        }
     }
 }
 
@@ -273,16 +331,17 @@ extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t 
     if (padded_entries == 0) return 0;
     if (dense == nullptr || row_ptr == nullptr || values == nullptr || deltas == nullptr)
         return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(values) & 1) ||
+    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(values) & 15) ||
         (reinterpret_cast<uintptr_t>(deltas) & 3))
         return MACKO_E_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
-    hipError_t e = hipMemsetAsync(values, 0, (size_t)padded_entries * 2, s);
+    // row-boundary nibbles are OR-ed in, so the nibble array starts from zero
+    hipError_t e = hipMemsetAsync(deltas, 0, (size_t)padded_entries / 2, s);
     if (e != hipSuccess) return (int)e;
-    e = hipMemsetAsync(deltas, 0, (size_t)padded_entries / 2, s);
-    if (e != hipSuccess) return (int)e;
+    if (rows == 0) return (int)hipMemsetAsync(values, 0, (size_t)padded_entries * 2, s);
     hipLaunchKernelGGL(fill_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
-                       (const uint16_t *)dense, rows, cols, row_ptr, (uint16_t *)values, (unsigned char *)deltas);
+                       (const uint16_t *)dense, rows, cols, row_ptr, (uint16_t *)values, (u32 *)deltas,
+                       (int)padded_entries);
     return (int)hipGetLastError();
 }
 
