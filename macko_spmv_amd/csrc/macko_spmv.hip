@@ -40,10 +40,12 @@ struct SpmvArgs {
     long long padded;       // P
     float alpha;
     float beta;
-    // split of the P stored entries and of the rows over the launch's waves, precomputed on the
-    // host so the kernel does no 64-bit division: wave w starts at w*q + min(w, rem)
+    // Precomputed on the host so the kernel does no 64-bit division.  The P stored entries are
+    // dealt to the launch's W waves as evenly as possible: wave w starts at w*q + min(w, rem).
+    // Where wave w's first row should be if all rows were equally long, floor(w*rows/W), is
+    // w*rows_q + ((w*rows_frac) >> 32) with rows_frac = floor((rows % W) * 2^32 / W).
     u32 entries_q, entries_rem;
-    u32 rows_q, rows_rem;
+    u32 rows_q, rows_frac;
 #ifdef MACKO_SPMV_TRACE
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif
@@ -364,8 +366,8 @@ spmv_stream_kernel(const SpmvArgs a)
     {
         target[0] = (int)even_split(gw, a.entries_q, a.entries_rem);  // < P < 2^31
         target[1] = (int)even_split(gw + 1, a.entries_q, a.entries_rem);
-        base[0] = probe_base((int)even_split(gw, a.rows_q, a.rows_rem), a.rows);
-        base[1] = probe_base((int)even_split(gw + 1, a.rows_q, a.rows_rem), a.rows);
+        base[0] = probe_base((int)(gw * a.rows_q + __umulhi(gw, a.rows_frac)), a.rows);
+        base[1] = probe_base((int)((gw + 1) * a.rows_q + __umulhi(gw + 1, a.rows_frac)), a.rows);
         int i0 = base[0] + lane, i1 = base[1] + lane;
         i0 = i0 <= a.rows ? i0 : a.rows;
         i1 = i1 <= a.rows ? i1 : a.rows;
@@ -632,7 +634,7 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
     a.entries_q = (u32)(a.padded / n_waves);
     a.entries_rem = (u32)(a.padded % n_waves);
     a.rows_q = (u32)a.rows / n_waves;
-    a.rows_rem = (u32)a.rows % n_waves;
+    a.rows_frac = (u32)(((unsigned long long)((u32)a.rows % n_waves) << 32) / n_waves);
     if (lds_bytes > 64 * 1024) {
         // one-time opt-in to more than 64 KiB of dynamic LDS, per device
         static bool done[64] = {};
