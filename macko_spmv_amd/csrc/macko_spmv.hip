@@ -101,12 +101,12 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
     for (int k = 0; k < 2; ++k) {
         const bool beyond = base[k] + lane > rows;
         const unsigned long long m = __ballot(beyond || window[k] >= target[k]);
-        if (m == 0) {  // everything probed is below the target
+        if (__builtin_expect(m == 0, 0)) {  // everything probed is below the target
             lo[k] = base[k] + 64 > rows ? rows : base[k] + 64;
             hi[k] = rows;
         } else {
             const int f = __builtin_ctzll(m);
-            if (f == 0) {  // the answer is at or before the window start
+            if (__builtin_expect(f == 0, 0)) {  // the answer is at or before the window start
                 lo[k] = 0;
                 hi[k] = base[k];
             } else {
@@ -114,7 +114,7 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
             }
         }
     }
-    while (lo[0] < hi[0] || lo[1] < hi[1]) {
+    while (__builtin_expect(lo[0] < hi[0] || lo[1] < hi[1], 0)) {
         int step[2], probe[2];
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
@@ -347,20 +347,10 @@ spmv_stream_kernel(const SpmvArgs a)
     (void)rs_x;
     const u32 lane16 = (u32)lane * 16, lane4 = (u32)lane * 4;
 
-    // ---- 1. x: everything beyond the two register pieces per thread, and unaligned or odd-length
-    //         x, is copied first (ordinary loads; done before any tracked load is issued) ---------
     const bool x_vec = (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
     const int x_nvec = x_vec ? a.cols >> 3 : 0;
-    if (X_LDS) {
-        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
-        for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
-        for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
-        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
-    }
 
-    // ---- 2. tracked loads, oldest first: row_ptr probes, x pieces ------------------------------------
+    // ---- 1. tracked loads, oldest first: row_ptr probes, x pieces ------------------------------------
     // probes: 64 consecutive row_ptr values around where my first / last row should be
     int target[2], base[2];
     {
@@ -384,6 +374,19 @@ spmv_stream_kernel(const SpmvArgs a)
         ring_issue<D, J>(lane16 + (fetch ? tile << (kTileShift + 1) : kNoTileValues),
                          lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas);
     };
+    // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
+    //         x, goes to LDS through ordinary loads (rare: more than 16384 columns, or an x that is
+    //         not 16-byte aligned) ------------------------------------------------------------------
+    if (X_LDS) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
+        if (__builtin_expect(x_nvec > kXRegs * BLOCK, 0))
+            for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
+        if (__builtin_expect((x_nvec << 3) < a.cols, 0))
+            for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
+        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
+        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
+    }
     MACKO_STAMP(1);
 
     // ---- 3. which rows are mine -----------------------------------------------------------------------
@@ -400,7 +403,7 @@ spmv_stream_kernel(const SpmvArgs a)
         const int rr = range[k];
         if (rr > 0 && rr <= a.rows) {
             int after, before;
-            if (rr - 1 >= base[k] && rr <= base[k] + 63) {
+            if (__builtin_expect(rr - 1 >= base[k] && rr <= base[k] + 63, 1)) {
                 after = __builtin_amdgcn_readlane(window[k], rr - base[k]);
                 before = __builtin_amdgcn_readlane(window[k], rr - 1 - base[k]);
             } else {
@@ -424,7 +427,7 @@ spmv_stream_kernel(const SpmvArgs a)
         return __builtin_amdgcn_readlane(win, r - win_base);
     };
     auto slide_window = [&](int r) {  // make rows r and r + 1 addressable
-        if (r < win_base || r + 1 > win_base + 63) {
+        if (__builtin_expect(r < win_base || r + 1 > win_base + 63, 0)) {
             win_base = r;
             win = load_row_window(a.row_ptr, a.rows, win_base, lane);
         }
@@ -442,11 +445,11 @@ spmv_stream_kernel(const SpmvArgs a)
     int r = row_first;
     int e0 = 0, e1 = 0, s_end = 0;
     u32 first_tile = 0, last_tile = 0;
-    if (have_work) {
+    if (__builtin_expect(have_work, 1)) {
         slide_window(r);
         e0 = row_start(r);
         e1 = row_start(r + 1);
-        while (e1 == e0) {
+        while (__builtin_expect(e1 == e0, 0)) {
             store_row(r, 0.f);
             ++r;
             if (r >= row_last) {
@@ -458,7 +461,7 @@ spmv_stream_kernel(const SpmvArgs a)
             e1 = row_start(r + 1);
         }
     }
-    if (have_work) {
+    if (__builtin_expect(have_work, 1)) {
         // end of my last owned row
         s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
         first_tile = (u32)e0 >> kTileShift;
@@ -475,7 +478,7 @@ spmv_stream_kernel(const SpmvArgs a)
     if (X_LDS) {
         u32x4 *d4 = reinterpret_cast<u32x4 *>(lds + kLdsFront);
         u32x4 x0, x1;
-        if (have_work) {
+        if (__builtin_expect(have_work, 1)) {
             x0 = xpiece_take<0, kTileLoads + 1>();
             x1 = xpiece_take<1, kTileLoads>();
         } else {
@@ -489,7 +492,7 @@ spmv_stream_kernel(const SpmvArgs a)
     }
     MACKO_STAMP(4);
 
-    if (!have_work) return;
+    if (__builtin_expect(!have_work, 0)) return;
 
     // ---- 6. stream ----------------------------------------------------------------------------------
     float acc0 = 0.f, acc1 = 0.f;
