@@ -71,8 +71,10 @@ int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols,
                              int32_t *row_ptr, void *stream);
 
 /*
- * Compressor, step 2 of 2.  Fills values [P] and deltas [P/2] (both fully written, tail
- * zero-filled) from `dense` and the row_ptr produced by step 1.  Asynchronous.
+ * Compressor, step 2 of 2.  Fills values [P] (16-byte aligned) and deltas [P/2] (4-byte
+ * aligned) from `dense` and the row_ptr produced by step 1; both arrays are fully written,
+ * tail zero-filled, whatever they held before.  P must be ceil(row_ptr[rows]/8)*8.
+ * Asynchronous.
  */
 int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
                             const int32_t *row_ptr, void *values, void *deltas,
