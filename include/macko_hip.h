@@ -81,6 +81,27 @@ int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
                             int64_t padded_entries, void *stream);
 
 /*
+ * int8 values variant.  Same arrays, except that `values` holds int8 [P] (8-byte aligned) and
+ * `dense` is a row-major int8 matrix.  The compressor pair replaces compress_rows_int8_cpu
+ * (src/macko_spmv/cuda/cpu_compressor.cuh:75-117), which differs from the fp16 one in keeping
+ * the padding entries behind a row's last non-zero; the products replace
+ * macko_spmv_int8<false> / <true> (src/macko_spmv/cuda/kernels.cuh:126-216; launched by
+ * c_benchmarking/benchmark.cu:106-118): y = fp16(alpha * sum float(value) * float(x[col])
+ * [+ beta * y]), fp32 accumulation.
+ */
+int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols,
+                            int32_t *row_ptr, void *stream);
+int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols,
+                           const int32_t *row_ptr, void *values, void *deltas,
+                           int64_t padded_entries, void *stream);
+int macko_spmv_i8f16(const void *values, const void *deltas, const int32_t *row_ptr,
+                     const void *x, void *y, int32_t rows, int32_t cols,
+                     int64_t padded_entries, void *stream);
+int macko_spmv_i8f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+                           const void *x, void *y, int32_t rows, int32_t cols,
+                           int64_t padded_entries, float alpha, float beta, void *stream);
+
+/*
  * Inverse of the compressor: writes the dense row-major fp16 matrix [rows, cols] (every
  * element written).  Uses the decode rule of the multiply kernel
  * (src/macko_spmv/cuda/kernels.cuh:97-103); the upstream package has no such function, it is

@@ -36,7 +36,7 @@ def _load_native():
     except OSError as exc:  # no silent fallback: the HIP path is the only path
         raise ImportError(
             f"macko_spmv_amd: cannot load its native libraries ({hip_path}, {torch_path}): {exc}. "
-            "Rebuild them with `python -m macko_spmv_amd._build`."
+            "Rebuild them with `python macko_spmv_amd/_build.py`."
         ) from exc
     return hip, hip_path, torch_path
 
@@ -52,6 +52,16 @@ def _multiply_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
 
 @torch.library.register_fake("macko_spmv::multiply_axpby")
 def _multiply_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C, alpha, beta):
+    return None
+
+
+@torch.library.register_fake("macko_spmv::multiply_int8")
+def _multiply_int8_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
+    return torch.empty((M_rows,), device=V.device, dtype=V.dtype)
+
+
+@torch.library.register_fake("macko_spmv::multiply_int8_axpby")
+def _multiply_int8_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C, alpha, beta):
     return None
 
 
@@ -112,6 +122,39 @@ def multiply_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):
         compressed_M[0], compressed_M[1], compressed_M[2], compressed_M[3], compressed_M[4], V, C,
         float(alpha), float(beta),
     )
+    return C
+
+
+def compress_int8(M):
+    """Dense int8 matrix -> (values int8[P], deltas uint8[P/2], row_indices int32[R+1], R, C).
+
+    The int8 twin of compress (compress_rows_int8_cpu, src/macko_spmv/cuda/cpu_compressor.cuh:75-117;
+    upstream has no Python entry for it).  Unlike the fp16 format it keeps the padding entries
+    behind a row's last non-zero.  Device routing as in compress.
+    """
+    assert M.is_contiguous()
+    if M.device.type in ("cuda", "cpu"):
+        return tuple(torch.ops.macko_spmv.compress_int8.default(M))
+    raise NotImplementedError()
+
+
+def multiply_int8(compressed_M, V):
+    """y = M @ V for an int8-compressed M and an fp16 V; fp32 accumulation, fp16 out
+    (macko_spmv_int8<false>, src/macko_spmv/cuda/kernels.cuh:126-216)."""
+    assert compressed_M[0].is_cuda
+    assert compressed_M[1].is_cuda
+    assert compressed_M[2].is_cuda
+    assert V.is_cuda
+    assert V.is_contiguous()
+    return torch.ops.macko_spmv.multiply_int8.default(*compressed_M[:5], V)
+
+
+def multiply_int8_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):
+    """In place C = alpha * (M @ V) + beta * C with int8 values (macko_spmv_int8<true>,
+    src/macko_spmv/cuda/kernels.cuh:208-211)."""
+    assert compressed_M[0].is_cuda and V.is_cuda and C.is_cuda
+    assert V.is_contiguous() and C.is_contiguous()
+    torch.ops.macko_spmv.multiply_int8_axpby.default(*compressed_M[:5], V, C, float(alpha), float(beta))
     return C
 
 

@@ -1,6 +1,6 @@
-// MACKO fp16 compressor and decompressor for gfx950 (wave64).
+// MACKO compressors (fp16 and int8 values) and fp16 decompressor for gfx950 (wave64).
 //
-// The format is restated from src/macko_spmv/cuda/cpu_compressor.cuh:6-73 of the upstream
+// The fp16 format is restated from src/macko_spmv/cuda/cpu_compressor.cuh:6-73 of the upstream
 // package as a per-column rule that needs no sequential walk:
 //   column x of a row stores an entry when its element is non-zero as a float (so -0.0 does
 //   not count and NaN does), or when x - p is a positive multiple of 16, p being the column
@@ -9,6 +9,9 @@
 //   non-zero are not stored.  A stored element keeps its bits (a padding entry keeps the sign
 //   of its zero); a NaN is stored as 0x7fff, the result of CUDA's float->half conversion that
 //   the upstream code routes every value through.
+//
+// The int8 format (compress_rows_int8_cpu, cpu_compressor.cuh:75-117) follows the same rule on
+// int8 elements, except that the padding entries after a row's last non-zero ARE stored.
 //
 // Pass 1 (count_rows_kernel + scan_rows_kernel) produces row_ptr; pass 2 (fill_rows_kernel)
 // writes values and nibbles.  One wave owns one row in both passes; lanes take 8 consecutive
@@ -23,33 +26,53 @@ constexpr int kRowsPerBlock = 4;              // waves per workgroup, one row ea
 constexpr int kBlock = kRowsPerBlock * kWave;
 constexpr int kNoColumn = (int)0x80000000;
 
-// 8 consecutive fp16 elements of a row, zero beyond `cols`.
-__device__ __forceinline__ u32x4 load8(const uint16_t *__restrict__ row, int col, int cols, bool vector_ok)
+// The two element formats.  A chunk is the 8 consecutive elements a lane handles per tile.
+struct Fp16Format {
+    typedef uint16_t Elem;
+    typedef u32x4 Chunk;                          // 8 halves
+    static constexpr bool kKeepTrailing = false;  // padding entries behind the last non-zero are dropped
+    static __device__ __forceinline__ u32 at(const Chunk &v, int i) { return (v[i >> 1] >> (16 * (i & 1))) & 0xffffu; }
+    static __device__ __forceinline__ void put(Chunk &v, int i, u32 bits) { v[i >> 1] |= bits << (16 * (i & 1)); }
+    // non-zero as a float: -0.0 is a zero, NaN is not
+    static __device__ __forceinline__ bool nonzero(u32 bits) { return (bits & 0x7fffu) != 0; }
+    // what is stored: the element itself, a NaN as 0x7fff
+    static __device__ __forceinline__ u32 stored(u32 bits) { return (bits & 0x7fffu) > 0x7c00u ? 0x7fffu : bits; }
+};
+struct Int8Format {
+    typedef unsigned char Elem;
+    typedef u32x2 Chunk;                         // 8 bytes
+    static constexpr bool kKeepTrailing = true;  // cpu_compressor.cuh:75-117 has no withdrawal step
+    static __device__ __forceinline__ u32 at(const Chunk &v, int i) { return (v[i >> 2] >> (8 * (i & 3))) & 0xffu; }
+    static __device__ __forceinline__ void put(Chunk &v, int i, u32 bits) { v[i >> 2] |= bits << (8 * (i & 3)); }
+    static __device__ __forceinline__ bool nonzero(u32 bits) { return bits != 0; }
+    static __device__ __forceinline__ u32 stored(u32 bits) { return bits; }
+};
+
+// 8 consecutive elements of a row, zero beyond `cols`.
+template <typename F>
+__device__ __forceinline__ typename F::Chunk load8(const typename F::Elem *__restrict__ row, int col, int cols,
+                                                   bool vector_ok)
 {
-    u32x4 v = {0, 0, 0, 0};
+    typename F::Chunk v = {};
     if (col + 8 <= cols && vector_ok) {
-        v = *reinterpret_cast<const u32x4 *>(row + col);
+        v = *reinterpret_cast<const typename F::Chunk *>(row + col);
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            u32 h = (col + i < cols) ? row[col + i] : 0u;
-            v[i >> 1] |= h << (16 * (i & 1));
+            const u32 h = (col + i < cols) ? (u32)row[col + i] : 0u;
+            F::put(v, i, h);
         }
     }
     return v;
 }
 
-__device__ __forceinline__ u32 half_at(const u32x4 &v, int i)
-{
-    return (v[i >> 1] >> (16 * (i & 1))) & 0xffffu;
-}
-
-// bit i set when element i is non-zero as a float
-__device__ __forceinline__ u32 nonzero_bits(const u32x4 &v)
+// bit i set when element i is non-zero
+template <typename F>
+__device__ __forceinline__ u32 nonzero_bits(const typename F::Chunk &v)
 {
     u32 m = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) m |= ((half_at(v, i) & 0x7fffu) != 0 ? 1u : 0u) << i;
+    for (int i = 0; i < 8; ++i) m |= (F::nonzero(F::at(v, i)) ? 1u : 0u) << i;
     return m;
 }
 
@@ -70,20 +93,23 @@ __device__ __forceinline__ int wave_sum_int(int x)
     return __builtin_amdgcn_readlane(wave_scan_inclusive(x), kWave - 1);
 }
 
-__global__ void __launch_bounds__(kBlock) count_rows_kernel(const uint16_t *__restrict__ dense, int rows,
+template <typename F>
+__global__ void __launch_bounds__(kBlock) count_rows_kernel(const typename F::Elem *__restrict__ dense, int rows,
                                                             int cols, int *__restrict__ counts)
 {
+    typedef typename F::Elem Elem;
+    typedef typename F::Chunk Chunk;
     const int lane = threadIdx.x & (kWave - 1);
     const int row = blockIdx.x * kRowsPerBlock + uniform(threadIdx.x >> 6);
     if (row >= rows) return;
-    const uint16_t *src = dense + (size_t)row * (size_t)cols;
-    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+    const Elem *src = dense + (size_t)row * (size_t)cols;
+    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & (sizeof(Chunk) - 1)) == 0;
     int carry = -1;  // column of the last non-zero seen in earlier passes
     int mine = 0;
     for (int c0 = 0; c0 < cols; c0 += kTile) {
         const int col = c0 + lane * kChunk;
-        const u32x4 v = load8(src, col, cols, vector_ok && col < cols);
-        const u32 nz = nonzero_bits(v);
+        const Chunk v = load8<F>(src, col, cols, vector_ok && col < cols);
+        const u32 nz = nonzero_bits<F>(v);
         const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
         int pass_last;
         int p = previous_nonzero(own_last, carry, lane, pass_last);
@@ -96,7 +122,8 @@ __global__ void __launch_bounds__(kBlock) count_rows_kernel(const uint16_t *__re
         }
         carry = pass_last > carry ? pass_last : carry;
     }
-    const int total = wave_sum_int(mine);
+    int total = wave_sum_int(mine);
+    if (F::kKeepTrailing) total += (cols - 1 - carry) >> 4;  // padding entries at carry+16, carry+32, ... < cols
     if (lane == 0) counts[row] = total;
 }
 
@@ -149,11 +176,14 @@ __device__ __forceinline__ void wave_lds_fence()
 // values and one 4-byte store of nibbles.  Groups cut by a row boundary are shared with the
 // neighbouring row's wave: their values go out as 2-byte stores and their nibbles are OR-ed
 // into the (zeroed) delta word.  `deltas` must be zero on entry; `values` need not be.
-__global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__restrict__ dense, int rows,
+template <typename F>
+__global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Elem *__restrict__ dense, int rows,
                                                            int cols, const int *__restrict__ row_ptr,
-                                                           uint16_t *__restrict__ values,
+                                                           typename F::Elem *__restrict__ values,
                                                            u32 *__restrict__ delta_words, int padded)
 {
+    typedef typename F::Elem Elem;
+    typedef typename F::Chunk Chunk;
     constexpr int kStage = kTile + 8;  // a tile's entries plus the carried part of a group
     __shared__ u32 stage_all[kRowsPerBlock][kStage];
     const int lane = threadIdx.x & (kWave - 1);
@@ -163,15 +193,15 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__res
     const int e0 = row_ptr[row];
     const int e1 = row_ptr[row + 1];
     u32 *stage = stage_all[wave];
-    u32x4 *value_groups = reinterpret_cast<u32x4 *>(values);
+    Chunk *value_groups = reinterpret_cast<Chunk *>(values);
 
     if (row == rows - 1) {  // the unused tail of the last 8-entry group
         for (int i = e1 + lane; i < padded; i += kWave) values[i] = 0;
     }
     if (e0 == e1) return;
 
-    const uint16_t *src = dense + (size_t)row * (size_t)cols;
-    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+    const Elem *src = dense + (size_t)row * (size_t)cols;
+    const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & (sizeof(Chunk) - 1)) == 0;
 
     // stage[i] holds output entry base + i; [lo, hi) is staged and not yet written out
     int base = e0 & ~7;
@@ -190,9 +220,9 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__res
             const int b = hi - 8 * g < 8 ? hi - 8 * g : 8;
             const int out = (base >> 3) + g;
             if (a == 0 && b == 8) {
-                u32x4 v;
+                Chunk v = {};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = (e[2 * i] & 0xffffu) | (e[2 * i + 1] << 16);
+                for (int i = 0; i < 8; ++i) F::put(v, i, e[i] & 0xffffu);
                 value_groups[out] = v;
                 delta_words[out] = pack_nibbles(e);
             } else {
@@ -200,7 +230,7 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__res
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     if (i >= a && i < b) {
-                        values[8 * (size_t)out + i] = (uint16_t)e[i];
+                        values[8 * (size_t)out + i] = (Elem)e[i];
                         keep |= 15u << (4 * i);
                     }
                 }
@@ -209,15 +239,15 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__res
         }
     };
 
-    u32x4 next = load8(src, lane * kChunk, cols, vector_ok && lane * kChunk < cols);
+    Chunk next = load8<F>(src, lane * kChunk, cols, vector_ok && lane * kChunk < cols);
     for (int c0 = 0; c0 < cols; c0 += kTile) {
         const int col = c0 + lane * kChunk;
-        const u32x4 v = next;
+        const Chunk v = next;
         if (c0 + kTile < cols) {
             const int ncol = col + kTile;
-            next = load8(src, ncol, cols, vector_ok && ncol < cols);
+            next = load8<F>(src, ncol, cols, vector_ok && ncol < cols);
         }
-        const u32 nz = nonzero_bits(v);
+        const u32 nz = nonzero_bits<F>(v);
         const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
         int pass_last;
         int p = previous_nonzero(own_last, carry, lane, pass_last);
@@ -246,9 +276,7 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const uint16_t *__res
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             if ((entry_bits & (1u << i)) && slot < n_new) {
-                u32 h = half_at(v, i);
-                h = (h & 0x7fffu) > 0x7c00u ? 0x7fffu : h;
-                stage[hi + slot] = h | (((nibbles >> (4 * i)) & 15u) << 16);
+                stage[hi + slot] = F::stored(F::at(v, i)) | (((nibbles >> (4 * i)) & 15u) << 16);
                 ++slot;
             }
         }
@@ -301,19 +329,22 @@ __global__ void __launch_bounds__(kBlock) decode_rows_kernel(const uint16_t *__r
 }  // namespace
 }  // namespace macko
 
-extern "C" int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
-                                        void *stream)
+namespace macko {
+namespace {
+
+template <typename F>
+int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr, void *stream)
 {
-    using namespace macko;
+    typedef typename F::Elem Elem;
     if (rows < 0 || cols < 0 || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
     if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
     if (rows > 0 && cols > 0 && dense == nullptr) return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(row_ptr) & 3))
+    if ((reinterpret_cast<uintptr_t>(dense) & (sizeof(Elem) - 1)) || (reinterpret_cast<uintptr_t>(row_ptr) & 3))
         return MACKO_E_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
     if (rows > 0) {
-        hipLaunchKernelGGL(count_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0,
-                           s, (const uint16_t *)dense, rows, cols, row_ptr + 1);
+        hipLaunchKernelGGL(count_rows_kernel<F>, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0,
+                           s, (const Elem *)dense, rows, cols, row_ptr + 1);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
@@ -321,28 +352,59 @@ extern "C" int macko_compress_f16_count(const void *dense, int32_t rows, int32_t
     return (int)hipGetLastError();
 }
 
-extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,
-                                       void *values, void *deltas, int64_t padded_entries, void *stream)
+template <typename F>
+int compress_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr, void *values,
+                  void *deltas, int64_t padded_entries, void *stream)
 {
-    using namespace macko;
+    typedef typename F::Elem Elem;
     if (rows < 0 || cols < 0 || padded_entries < 0 || padded_entries % kChunk != 0)
         return MACKO_E_INVALID_ARGUMENT;
     if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
     if (padded_entries == 0) return 0;
     if (dense == nullptr || row_ptr == nullptr || values == nullptr || deltas == nullptr)
         return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(dense) & 1) || (reinterpret_cast<uintptr_t>(values) & 15) ||
+    if ((reinterpret_cast<uintptr_t>(dense) & (sizeof(Elem) - 1)) ||
+        (reinterpret_cast<uintptr_t>(values) & (sizeof(typename F::Chunk) - 1)) ||
         (reinterpret_cast<uintptr_t>(deltas) & 3))
         return MACKO_E_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
     // row-boundary nibbles are OR-ed in, so the nibble array starts from zero
     hipError_t e = hipMemsetAsync(deltas, 0, (size_t)padded_entries / 2, s);
     if (e != hipSuccess) return (int)e;
-    if (rows == 0) return (int)hipMemsetAsync(values, 0, (size_t)padded_entries * 2, s);
-    hipLaunchKernelGGL(fill_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
-                       (const uint16_t *)dense, rows, cols, row_ptr, (uint16_t *)values, (u32 *)deltas,
+    if (rows == 0) return (int)hipMemsetAsync(values, 0, (size_t)padded_entries * sizeof(Elem), s);
+    hipLaunchKernelGGL(fill_rows_kernel<F>, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
+                       (const Elem *)dense, rows, cols, row_ptr, (Elem *)values, (u32 *)deltas,
                        (int)padded_entries);
     return (int)hipGetLastError();
+}
+
+}  // namespace
+}  // namespace macko
+
+extern "C" int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                        void *stream)
+{
+    return macko::compress_count<macko::Fp16Format>(dense, rows, cols, row_ptr, stream);
+}
+
+extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,
+                                       void *values, void *deltas, int64_t padded_entries, void *stream)
+{
+    return macko::compress_fill<macko::Fp16Format>(dense, rows, cols, row_ptr, values, deltas, padded_entries,
+                                                   stream);
+}
+
+extern "C" int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                       void *stream)
+{
+    return macko::compress_count<macko::Int8Format>(dense, rows, cols, row_ptr, stream);
+}
+
+extern "C" int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,
+                                      void *values, void *deltas, int64_t padded_entries, void *stream)
+{
+    return macko::compress_fill<macko::Int8Format>(dense, rows, cols, row_ptr, values, deltas, padded_entries,
+                                                   stream);
 }
 
 extern "C" int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr, int32_t rows,

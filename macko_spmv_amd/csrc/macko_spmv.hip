@@ -30,7 +30,7 @@ constexpr int kTileShift = 9;   // log2(kTile)
 constexpr int kXRegs = 2;       // 16-byte pieces of x a thread fetches with tracked loads
 
 struct SpmvArgs {
-    const u32 *values;      // fp16 pairs
+    const u32 *values;      // fp16 pairs (or int8 quads for the int8 variant)
     const u32 *deltas;      // 8 nibbles per word
     const int *row_ptr;
     const uint16_t *x;
@@ -142,10 +142,18 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
     out[1] = lo[1];
 }
 
-// 128-bit mask helpers: keep halves [from, 8) / [0, upto) of a 4-dword vector and the matching
-// nibbles.  `from` / `upto` are wave-uniform, so the masks are built on the scalar unit.
+// Mask helpers: keep values [from, 8) / [0, upto) of a lane's 8 values (VB bytes each) and the
+// matching nibbles.  `from` / `upto` are wave-uniform, so the masks are built on the scalar unit.
+template <int VB>
 __device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)  // 1 <= from <= 7
 {
+    if (VB == 1) {  // 8 one-byte values in v.x, v.y
+        const unsigned long long m = ~0ull << (8 * from);
+        v.x &= (u32)m;
+        v.y &= (u32)(m >> 32);
+        d &= ~0u << (4 * from);
+        return;
+    }
     const unsigned long long lo = from < 4 ? (~0ull << (16 * from)) : 0ull;
     const unsigned long long hi = from < 4 ? ~0ull : (~0ull << (16 * (from - 4)));
     v.x &= (u32)lo;
@@ -155,8 +163,16 @@ __device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)  // 1 <= f
     d &= ~0u << (4 * from);
 }
 
+template <int VB>
 __device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= upto <= 7
 {
+    if (VB == 1) {
+        const unsigned long long m = (1ull << (8 * upto)) - 1;
+        v.x &= (u32)m;
+        v.y &= (u32)(m >> 32);
+        d &= (1u << (4 * upto)) - 1;
+        return;
+    }
     const unsigned long long lo = upto < 4 ? ((1ull << (16 * upto)) - 1) : ~0ull;
     const unsigned long long hi = upto <= 4 ? 0ull : ((1ull << (16 * (upto - 4))) - 1);
     v.x &= (u32)lo;
@@ -251,11 +267,24 @@ __device__ __forceinline__ u32x4 xpiece_take()
                  "\n\tv_mov_b32 %3, " E "\n\tv_mov_b32 %4, " DREG                                               \
                  : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w), "=v"(d) : "n"(N) : "memory")
 
-template <int D, int J>
+#define MACKO_RING_ISSUE_I8(VREGS, DREG, CLOBBERS)                                                         \
+    asm volatile("buffer_load_dwordx2 " VREGS ", %0, %2, 0 offen\n\tbuffer_load_dword " DREG ", %1, %3, 0 offen" \
+                 ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
+                 : "memory", CLOBBERS)
+
+// VB = bytes per stored value: 2 (fp16, 16 bytes per lane and tile) or 1 (int8, 8 bytes per lane
+// and tile, which land in the first two registers of the slot).
+template <int D, int J, int VB>
 __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
                                            const u32x4 &buf_deltas)
 {
     static_assert(D == 1 || D == 2 || D == 4 || D == 8 || D == 16, "ring depth");
+    static_assert(VB == 2 || (VB == 1 && D == 2), "the int8 ring exists at depth 2 only");
+    if (VB == 1) {
+        if (J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v96", MACKO_FIXED_CLOBBERS_4);
+        if (J == 1) MACKO_RING_ISSUE_I8("v[92:93]", "v97", MACKO_FIXED_CLOBBERS_4);
+        return;
+    }
     if (D == 1 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v92", MACKO_FIXED_CLOBBERS_4);
     if (D == 2 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v96", MACKO_FIXED_CLOBBERS_4);
     if (D == 2 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v97", MACKO_FIXED_CLOBBERS_4);
@@ -324,7 +353,7 @@ __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
     if (D == 16 && J == 14) MACKO_RING_TAKE("v144", "v145", "v146", "v147", "v166");
     if (D == 16 && J == 15) MACKO_RING_TAKE("v148", "v149", "v150", "v151", "v167");
 }
-template <int BLOCK, int D, bool X_LDS, bool AXPBY>
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
@@ -339,13 +368,13 @@ spmv_stream_kernel(const SpmvArgs a)
     MACKO_STAMP(0);
 
 
-    const u32x4 buf_values = make_buffer(a.values, (u32)(a.padded * 2));
+    const u32x4 buf_values = make_buffer(a.values, (u32)(a.padded * VB));
     const u32x4 buf_deltas = make_buffer(a.deltas, (u32)(a.padded / 2));
     const u32x4 buf_rows = make_buffer(a.row_ptr, ((u32)a.rows + 1) * 4);
     const __amdgpu_buffer_rsrc_t rs_x =
         __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.cols * 2, 0x00020000);
     (void)rs_x;
-    const u32 lane16 = (u32)lane * 16, lane4 = (u32)lane * 4;
+    const u32 lane_values = (u32)lane * (kChunk * VB), lane4 = (u32)lane * 4;
 
     const bool x_vec = (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
     const int x_nvec = x_vec ? a.cols >> 3 : 0;
@@ -371,7 +400,7 @@ spmv_stream_kernel(const SpmvArgs a)
     }
     auto issue_slot = [&](auto slot, u32 tile, bool fetch) {
         constexpr int J = decltype(slot)::value;
-        ring_issue<D, J>(lane16 + (fetch ? tile << (kTileShift + 1) : kNoTileValues),
+        ring_issue<D, J, VB>(lane_values + (fetch ? tile * (u32)(kTile * VB) : kNoTileValues),
                          lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas);
     };
     // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
@@ -524,12 +553,17 @@ spmv_stream_kernel(const SpmvArgs a)
                 xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
             }
 #endif
-            const u32 w = vv[k >> 1];
-            const uint16_t mb = (k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+            float m;
+            if (VB == 2) {
+                const u32 w = vv[k >> 1];
+                m = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+            } else {
+                m = (float)((int)(vv[k >> 2] << (24 - 8 * (k & 3))) >> 24);  // sign-extended byte k
+            }
             if (k & 1)
-                acc1 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc1);
+                acc1 = __builtin_fmaf(m, half_bits_to_float(xb), acc1);
             else
-                acc0 = __builtin_fmaf(half_bits_to_float(mb), half_bits_to_float(xb), acc0);
+                acc0 = __builtin_fmaf(m, half_bits_to_float(xb), acc0);
         }
     };
 
@@ -563,8 +597,8 @@ spmv_stream_kernel(const SpmvArgs a)
         u32x4 vv = vj;
         u32 dd = dj;
         const bool active = lane >= l0 && lane <= l1;
-        if (q0 != 0 && lane == l0) mask_from(vv, dd, q0);
-        if (q1 != 0 && lane == l1) mask_upto(vv, dd, q1);
+        if (q0 != 0 && lane == l0) mask_from<VB>(vv, dd, q0);
+        if (q1 != 0 && lane == l1) mask_upto<VB>(vv, dd, q1);
         u32 step = __builtin_amdgcn_udot8(dd, 0x22222222u, 16u, false);
         step = active ? step : 0u;
         const u32 incl = (u32)wave_scan_inclusive((int)step);
@@ -629,10 +663,10 @@ __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
-template <int BLOCK, int D, bool X_LDS, bool AXPBY>
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2>
 int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY>;
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
     a.entries_q = (u32)(a.padded / n_waves);
     a.entries_rem = (u32)(a.padded % n_waves);
@@ -663,7 +697,7 @@ struct Tuning {
 };
 Tuning g_tuning = {0, 0, 0};
 
-template <bool AXPBY>
+template <bool AXPBY, int VB = 2>
 int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 {
     if (a.rows == 0) return 0;
@@ -692,7 +726,13 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     if (grid < 1) grid = 1;
 
     const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
-    if (lds_need > (size_t)info.max_lds_bytes) return launch_stream<1024, 2, false, AXPBY>(a, (int)grid, 0, stream);
+    if (lds_need > (size_t)info.max_lds_bytes)
+        return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
+    if (VB == 1) {  // int8 values: the default launch shape only
+        if (block == 1024 && depth == 2)
+            return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_need, stream);
+        return MACKO_E_INVALID_ARGUMENT;
+    }
 #define MACKO_CASE(B, D_) \
     if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
     MACKO_CASE(1024, 2)
@@ -710,7 +750,7 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 }
 
 int check_spmv_args(const void *values, const void *deltas, const int32_t *row_ptr, const void *x, void *y,
-                    int32_t rows, int32_t cols, int64_t padded)
+                    int32_t rows, int32_t cols, int64_t padded, int value_bytes = 2)
 {
     if (rows < 0 || cols < 0 || padded < 0) return MACKO_E_INVALID_ARGUMENT;
     if (padded % kChunk != 0) return MACKO_E_INVALID_ARGUMENT;
@@ -718,7 +758,8 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
     if (rows > 0 && (row_ptr == nullptr || y == nullptr)) return MACKO_E_INVALID_ARGUMENT;
     if (padded > 0 && (values == nullptr || deltas == nullptr || x == nullptr || cols == 0))
         return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(values) & 15) || (reinterpret_cast<uintptr_t>(deltas) & 3) ||
+    if ((reinterpret_cast<uintptr_t>(values) & (uintptr_t)(8 * value_bytes - 1)) ||
+        (reinterpret_cast<uintptr_t>(deltas) & 3) ||
         (reinterpret_cast<uintptr_t>(row_ptr) & 3) || (reinterpret_cast<uintptr_t>(x) & 1) ||
         (reinterpret_cast<uintptr_t>(y) & 1))
         return MACKO_E_INVALID_ARGUMENT;
@@ -768,4 +809,36 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     a.trace = nullptr;
 #endif
     return spmv_dispatch<true>(a, as_stream(stream));
+}
+
+// int8 values x fp16 vector (macko_spmv_int8, src/macko_spmv/cuda/kernels.cuh:126-216).
+extern "C" int macko_spmv_i8f16(const void *values, const void *deltas, const int32_t *row_ptr, const void *x,
+                                void *y, int32_t rows, int32_t cols, int64_t padded_entries, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries, 1);
+    if (rc != 0) return rc;
+    SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
+               rows,                cols,                padded_entries, 1.0f,          0.0f,
+               0,                   0,                   0,              0};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = nullptr;
+#endif
+    return spmv_dispatch<false, 1>(a, as_stream(stream));
+}
+
+extern "C" int macko_spmv_i8f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+                                      const void *x, void *y, int32_t rows, int32_t cols,
+                                      int64_t padded_entries, float alpha, float beta, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries, 1);
+    if (rc != 0) return rc;
+    SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
+               rows,                cols,                padded_entries, alpha,         beta,
+               0,                   0,                   0,              0};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = nullptr;
+#endif
+    return spmv_dispatch<true, 1>(a, as_stream(stream));
 }

@@ -81,16 +81,18 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_on_dev
     const int64_t rows = M.size(0), cols = M.size(1);
     TORCH_CHECK(rows * cols < (1ll << 31), "matrix too large: rows * cols must stay below 2^31");
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const bool int8 = M.dtype() == at::kChar;
     at::Tensor row_ptr = at::empty({rows + 1}, M.options().dtype(at::kInt));
-    check_rc(macko_compress_f16_count(M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(),
-                                      (void *)stream),
+    check_rc((int8 ? macko_compress_i8_count : macko_compress_f16_count)(
+                 M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(), (void *)stream),
              "compress (count)");
     const int64_t n = row_ptr[rows].item<int>();  // one 4-byte read-back; sizes the outputs
     const int64_t padded = (n + 7) / 8 * 8;
     at::Tensor values = at::empty({padded}, M.options());
     at::Tensor deltas = at::empty({padded / 2}, M.options().dtype(at::kByte));
-    check_rc(macko_compress_f16_fill(M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(),
-                                     values.data_ptr(), deltas.data_ptr(), padded, (void *)stream),
+    check_rc((int8 ? macko_compress_i8_fill : macko_compress_f16_fill)(
+                 M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(), values.data_ptr(),
+                 deltas.data_ptr(), padded, (void *)stream),
              "compress (fill)");
     return std::make_tuple(values, deltas, row_ptr, rows, cols);
 }
@@ -120,6 +122,78 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_cpu(co
                            std::get<3>(out), std::get<4>(out));
 }
 
+// int8 twins (compress_rows_int8_cpu, src/macko_spmv/cuda/cpu_compressor.cuh:75-117, and
+// macko_spmv_int8, src/macko_spmv/cuda/kernels.cuh:126-216; upstream exposes them only in its C
+// benchmark, c_benchmarking/benchmark.cu:106-118).
+std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_int8_hip(const at::Tensor &M)
+{
+    TORCH_CHECK(M.dtype() == at::kChar, "M must be torch.int8");
+    TORCH_CHECK(M.dim() == 2, "M must be a matrix");
+    TORCH_CHECK(M.is_contiguous(), "M must be contiguous");
+    return compress_on_device(M);
+}
+
+std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_int8_cpu(const at::Tensor &M)
+{
+    TORCH_CHECK(M.dtype() == at::kChar, "M must be torch.int8");
+    TORCH_CHECK(M.dim() == 2, "M must be a matrix");
+    TORCH_CHECK(M.is_contiguous(), "M must be contiguous");
+    int n_dev = 0;
+    TORCH_CHECK(hipGetDeviceCount(&n_dev) == hipSuccess && n_dev > 0,
+                "macko_spmv: compress needs an AMD GPU (the compressor is a HIP kernel; there is no CPU path)");
+    auto out = compress_on_device(M.to(at::Device(at::kCUDA, c10::hip::current_device())));
+    return std::make_tuple(std::get<0>(out).cpu(), std::get<1>(out).cpu(), std::get<2>(out).cpu(),
+                           std::get<3>(out), std::get<4>(out));
+}
+
+void check_int8_operands(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                         int64_t M_rows, int64_t M_cols, const at::Tensor &V)
+{
+    TORCH_CHECK(M_values.dtype() == at::kChar, "M must be torch.int8");
+    TORCH_CHECK(V.dtype() == at::kHalf, "V must be torch.half");
+    TORCH_CHECK(M_deltas.dtype() == at::kByte, "M_deltas must be torch.uint8");
+    TORCH_CHECK(M_row_indices.dtype() == at::kInt, "M_row_indices must be torch.int32");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda(),
+                "all tensors must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
+                    V.is_contiguous(),
+                "all tensors must be contiguous");
+    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
+    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
+    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+    TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
+}
+
+at::Tensor multiply_int8_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                             const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &V)
+{
+    check_int8_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols, V);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    at::Tensor C = at::empty({M_rows}, V.options());
+    check_rc(macko_spmv_i8f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                              V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols, M_values.numel(),
+                              (void *)stream),
+             "multiply_int8");
+    return C;
+}
+
+// C = alpha * (M @ V) + beta * C, in place on C.
+void multiply_int8_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                             const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &V,
+                             at::Tensor C, double alpha, double beta)
+{
+    check_int8_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols, V);
+    TORCH_CHECK(C.dtype() == at::kHalf && C.is_cuda() && C.is_contiguous() && C.numel() >= M_rows,
+                "C must be a contiguous torch.half GPU tensor with at least M_rows elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    check_rc(macko_spmv_i8f16_axpby(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                    V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols, M_values.numel(),
+                                    (float)alpha, (float)beta, (void *)stream),
+             "multiply_int8_axpby");
+}
+
 at::Tensor decompress_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
                           int64_t M_rows, int64_t M_cols)
 {
@@ -145,6 +219,11 @@ TORCH_LIBRARY(macko_spmv, m)
     m.def("multiply_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
           "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
     m.def("compress(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
+    m.def("compress_int8(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
+    m.def("multiply_int8(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V) -> Tensor");
+    m.def("multiply_int8_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
     m.def("decompress(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols) -> Tensor");
 }
 
@@ -153,10 +232,14 @@ TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
     m.impl("multiply", &multiply_hip);
     m.impl("multiply_axpby", &multiply_axpby_hip);
     m.impl("compress", &compress_hip);
+    m.impl("compress_int8", &compress_int8_hip);
+    m.impl("multiply_int8", &multiply_int8_hip);
+    m.impl("multiply_int8_axpby", &multiply_int8_axpby_hip);
     m.impl("decompress", &decompress_hip);
 }
 
 TORCH_LIBRARY_IMPL(macko_spmv, CPU, m)
 {
     m.impl("compress", &compress_cpu);
+    m.impl("compress_int8", &compress_int8_cpu);
 }

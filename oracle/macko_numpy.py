@@ -1,4 +1,4 @@
-"""Closed-form NumPy statement of the MACKO fp16 format.  TEST INFRASTRUCTURE ONLY.
+"""Closed-form NumPy statements of the MACKO formats (fp16, int8).  TEST INFRASTRUCTURE ONLY.
 
 An independent second statement of what the upstream compressor emits
 (src/macko_spmv/cuda/cpu_compressor.cuh:6-73), used to cross-check the sequential C
@@ -56,6 +56,38 @@ def compress_closed_form(dense_bits):
         pad_col = prev[owner] + 16 * j
         pad_slot = pos[owner] - pads[owner] + (j - 1)
         values[pad_slot] = dense_bits[nz_r[owner], pad_col]
+    deltas = (nibbles[0::2] | (nibbles[1::2] << 4)).astype(np.uint8)
+    return values, deltas, row_ptr.astype(np.int32), n
+
+
+def compress_int8_closed_form(dense):
+    """int8 [R, C] -> (values int8 [P], deltas uint8 [P//2], row_ptr int32 [R+1], n).
+
+    Per-column statement of compress_rows_int8_cpu (cpu_compressor.cuh:75-117): with p the column
+    of the previous non-zero of the row (-1 before the first), column x stores an entry when its
+    element is non-zero, or when x - p is a positive multiple of 16 (a padding entry, nibble 15,
+    value 0).  A non-zero carries nibble (x - p - 1) & 15.  Unlike the fp16 format the padding
+    entries behind the last non-zero of a row stay.
+    """
+    dense = np.ascontiguousarray(dense, dtype=np.int8)
+    rows, cols = dense.shape
+    nz = dense != 0
+    col_idx = np.broadcast_to(np.arange(cols, dtype=np.int64), (rows, cols))
+    last_nz_incl = np.maximum.accumulate(np.where(nz, col_idx, -1), axis=1)
+    prev = np.full((rows, cols), -1, dtype=np.int64)
+    prev[:, 1:] = last_nz_incl[:, :-1]
+    dist = col_idx - prev
+    is_entry = nz | (dist % 16 == 0)
+    nib = np.where(nz, (dist - 1) & 15, 15).astype(np.uint8)
+    row_counts = is_entry.sum(axis=1)
+    row_ptr = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(row_counts, out=row_ptr[1:])
+    n = int(row_ptr[-1])
+    padded = (n + 7) // 8 * 8
+    nibbles = np.zeros(padded, dtype=np.uint8)
+    values = np.zeros(padded, dtype=np.int8)
+    nibbles[:n] = nib[is_entry]  # boolean indexing walks row-major
+    values[:n] = dense[is_entry]
     deltas = (nibbles[0::2] | (nibbles[1::2] << 4)).astype(np.uint8)
     return values, deltas, row_ptr.astype(np.int32), n
 

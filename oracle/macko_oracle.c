@@ -20,6 +20,17 @@
  *                               two known-answer vectors decoded by hand.
  *   macko_oracle_spmv_f16       pinned against a dense fp64 mat-vec (textbook
  *                               reduction) within the fp16 tolerance the tests state.
+ *   macko_oracle_compress_i8    the upstream tests hold no int8 vector.  Pinned by: an
+ *                               independent closed-form statement (macko_numpy.py); the
+ *                               special case that reduces to the fp16 compressor (rows whose
+ *                               last column is non-zero have no trailing padding entries, so
+ *                               row_ptr and nibbles must equal those of the known-answer-pinned
+ *                               fp16 compressor on the same non-zero pattern); format
+ *                               invariants; compress->decode round trips; a brute-force
+ *                               entry count.
+ *   macko_oracle_spmv_i8        pinned against a dense fp64 mat-vec within the fp16
+ *                               tolerance, and by exact agreement with a float64 product
+ *                               taken from the decoded arrays.
  *
  * Plain C99, no dependencies beyond libc/libm.  Half precision is handled as raw
  * uint16_t bit patterns so the file builds with any gcc.
@@ -267,5 +278,96 @@ void macko_oracle_dense_gemv_f16(const uint16_t *dense, const uint16_t *x, uint1
         for (int32_t c = 0; c < cols; ++c)
             acc = fmaf(half_bits_to_float(row[c]), half_bits_to_float(x[c]), acc);
         y[r] = float_to_half_bits(acc);
+    }
+}
+
+/* ---- int8 values variant --------------------------------------------------------------- */
+
+/*
+ * Compress a dense row-major int8 matrix.  Follows compress_rows_int8_cpu
+ * (src/macko_spmv/cuda/cpu_compressor.cuh:75-117): the same walk as the fp16 compressor
+ * (entry when the element is non-zero or 15 zeros have been skipped, :94-110), but the
+ * padding entries behind a row's last non-zero are KEPT (there is no withdrawal step), so an
+ * all-zero row of C columns stores C/16 padding entries.  row_ptr[r+1] is the running count
+ * (:111); arrays end at the count rounded up to a multiple of 8 (:113-117), zero filled
+ * (calloc, :82-83).  Same capacity / return convention as macko_oracle_compress_f16.
+ */
+int64_t macko_oracle_compress_i8(const int8_t *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                 int8_t *values, uint8_t *deltas, int64_t capacity, int64_t *padded)
+{
+    int64_t n = 0;
+    row_ptr[0] = 0;
+    for (int32_t r = 0; r < rows; ++r) {
+        const int8_t *row = dense + (size_t)r * (size_t)cols;
+        unsigned gap = 0;
+        for (int32_t c = 0; c < cols; ++c) {
+            if (row[c] != 0 || gap == MACKO_GAP_LIMIT) {
+                if (n >= capacity)
+                    return -1;
+                nibble_store(deltas, n, gap);
+                values[n] = row[c];
+                ++n;
+                gap = 0;
+            } else {
+                ++gap;
+            }
+        }
+        row_ptr[r + 1] = (int32_t)n;
+    }
+    int64_t p = (n + MACKO_CHUNK - 1) / MACKO_CHUNK * MACKO_CHUNK;
+    if (p > capacity)
+        return -1;
+    for (int64_t j = n; j < p; ++j) {
+        nibble_store(deltas, j, 0);
+        values[j] = 0;
+    }
+    if (padded)
+        *padded = p;
+    return n;
+}
+
+/* Decode of the int8 arrays: the column rule of macko_spmv_int8
+ * (src/macko_spmv/cuda/kernels.cuh:196-197), identical to the fp16 one. */
+int macko_oracle_decode_i8(const int8_t *values, const uint8_t *deltas, const int32_t *row_ptr,
+                           int32_t rows, int32_t cols, int8_t *dense)
+{
+    memset(dense, 0, (size_t)rows * (size_t)cols);
+    for (int32_t r = 0; r < rows; ++r) {
+        int64_t col = -1;
+        for (int64_t j = row_ptr[r]; j < row_ptr[r + 1]; ++j) {
+            col += (int64_t)nibble_load(deltas, j) + 1;
+            if (col >= cols)
+                return -1;
+            dense[(size_t)r * (size_t)cols + (size_t)col] = values[j];
+        }
+    }
+    return 0;
+}
+
+/*
+ * y = fp16(alpha * (M x) [+ beta * y]) for int8 values and an fp16 vector.  Follows
+ * macko_spmv_int8<reuse_value_from_c> (src/macko_spmv/cuda/kernels.cuh:126-216): fp32
+ * accumulator over float(value) * float(x[col]) (:198-202), column clamped to [0, cols-1]
+ * (:199-200), result rounded to fp16 (:208-215).  Summed left to right (the upstream order is
+ * lane-interleaved; the parity bar is tolerance based).
+ */
+void macko_oracle_spmv_i8(const int8_t *values, const uint8_t *deltas, const int32_t *row_ptr,
+                          const uint16_t *x, uint16_t *y, int32_t rows, int32_t cols, float alpha,
+                          float beta, int use_beta)
+{
+    for (int32_t r = 0; r < rows; ++r) {
+        float acc = 0.0f;
+        int64_t col = -1;
+        for (int64_t j = row_ptr[r]; j < row_ptr[r + 1]; ++j) {
+            col += (int64_t)nibble_load(deltas, j) + 1;
+            int64_t cc = col >= cols ? cols - 1 : col;
+            if (cc < 0)
+                cc = 0;
+            acc = fmaf((float)values[j], half_bits_to_float(x[cc]), acc);
+        }
+        float out = alpha * acc;
+        if (use_beta)
+            out += beta * half_bits_to_float(y[r]);
+        y[r] = float_to_half_bits(out);
     }
 }

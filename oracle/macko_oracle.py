@@ -40,6 +40,12 @@ def _load():
     lib.macko_oracle_spmv_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, f32, f32, ctypes.c_int]
     lib.macko_oracle_dense_gemv_f16.restype = None
     lib.macko_oracle_dense_gemv_f16.argtypes = [vp, vp, vp, i32, i32]
+    lib.macko_oracle_compress_i8.restype = i64
+    lib.macko_oracle_compress_i8.argtypes = [vp, i32, i32, vp, vp, vp, i64, ctypes.POINTER(i64)]
+    lib.macko_oracle_decode_i8.restype = ctypes.c_int
+    lib.macko_oracle_decode_i8.argtypes = [vp, vp, vp, i32, i32, vp]
+    lib.macko_oracle_spmv_i8.restype = None
+    lib.macko_oracle_spmv_i8.argtypes = [vp, vp, vp, vp, vp, i32, i32, f32, f32, ctypes.c_int]
     lib.macko_oracle_float_to_half.restype = ctypes.c_uint16
     lib.macko_oracle_float_to_half.argtypes = [f32]
     lib.macko_oracle_half_to_float.restype = f32
@@ -104,6 +110,49 @@ def spmv(values, deltas, row_ptr, rows, cols, x_bits, alpha=1.0, beta=None, y_bi
     y = np.zeros(rows, dtype=np.uint16) if y_bits is None else _u16(y_bits).copy()
     lib.macko_oracle_spmv_f16(_p(values), _p(deltas), _p(row_ptr), _p(x_bits), _p(y), rows, cols,
                               float(alpha), 0.0 if beta is None else float(beta), 0 if beta is None else 1)
+    return y
+
+
+def compress_int8(dense):
+    """int8 [R, C] -> (values int8 [P], deltas uint8 [P//2], row_ptr int32 [R+1], n)."""
+    lib = _load()
+    dense = np.ascontiguousarray(dense, dtype=np.int8)
+    rows, cols = dense.shape
+    cap = rows * cols + 8
+    values = np.zeros(cap, dtype=np.int8)
+    deltas = np.zeros(cap // 2, dtype=np.uint8)
+    row_ptr = np.zeros(rows + 1, dtype=np.int32)
+    padded = ctypes.c_int64(0)
+    n = lib.macko_oracle_compress_i8(_p(dense), rows, cols, _p(row_ptr), _p(values), _p(deltas), cap,
+                                     ctypes.byref(padded))
+    assert n >= 0
+    p = padded.value
+    return values[:p].copy(), deltas[: p // 2].copy(), row_ptr, int(n)
+
+
+def decode_int8(values, deltas, row_ptr, rows, cols):
+    lib = _load()
+    values = np.ascontiguousarray(values, dtype=np.int8)
+    deltas = np.ascontiguousarray(deltas, dtype=np.uint8)
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    dense = np.zeros((rows, cols), dtype=np.int8)
+    rc = lib.macko_oracle_decode_i8(_p(values), _p(deltas), _p(row_ptr), rows, cols, _p(dense))
+    if rc != 0:
+        raise ValueError("an entry decodes to a column outside the matrix")
+    return dense
+
+
+def spmv_int8(values, deltas, row_ptr, rows, cols, x_bits, alpha=1.0, beta=None, y_bits=None):
+    """int8 values x fp16 vector, fp32 accumulate, fp16 bits out (uint16 [rows])."""
+    lib = _load()
+    values = np.ascontiguousarray(values, dtype=np.int8)
+    deltas = np.ascontiguousarray(deltas, dtype=np.uint8)
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    x_bits = _u16(x_bits).reshape(-1)
+    assert x_bits.size >= cols
+    y = np.zeros(rows, dtype=np.uint16) if y_bits is None else _u16(y_bits).copy()
+    lib.macko_oracle_spmv_i8(_p(values), _p(deltas), _p(row_ptr), _p(x_bits), _p(y), rows, cols,
+                             float(alpha), 0.0 if beta is None else float(beta), 0 if beta is None else 1)
     return y
 
 
