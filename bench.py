@@ -199,6 +199,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
     ap.add_argument("--no-compress", action="store_true", help="skip the compressor timing")
+    ap.add_argument("--no-int8", action="store_true", help="skip the int8-values variant timing")
     ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
     ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
                     help="llama = the headline workload; large / skew = the other shape families")
@@ -324,6 +325,32 @@ def main():
             })
             log(per_case[-1])
 
+    # ---- int8 values variant on the same sparsity patterns (densities 0.1 and 0.5 only) ------------
+    int8_cases = []
+    if not args.no_int8:
+        for c in cases:
+            if c["density"] not in (0.1, 0.5):
+                continue
+            W = c["W"]
+            q = torch.round(W.float() * (127.0 / W.float().abs().max().item()))
+            q = torch.where((q == 0) & (W != 0), torch.sign(W.float()), q).to(torch.int8)  # keep the pattern
+            c8 = mk.compress_int8(q)
+            del q
+            nbytes = 1.5 * c8[0].numel() + 4 * (c["rows"] + 1) + 2 * c["cols"] + 2 * c["rows"]
+            n_copies = max(2, min(256, int(1.0e9 // nbytes) + 1))
+            copies = [c8] + [clone_compressed(c8) for _ in range(n_copies - 1)]
+            t8, _ = time_graph(torch, lambda: [mk.multiply_int8(cc, c["x"]) for cc in copies], args.case_replays)
+            t8 /= len(copies)
+            del copies
+            dense_us = next((p["dense_us"] for p in per_case
+                             if p["shape"] == f"{c['rows']}x{c['cols']}" and p["density"] == c["density"]), None)
+            int8_cases.append({
+                "shape": f"{c['rows']}x{c['cols']}", "density": c["density"], "us": round(t8 * 1e6, 2),
+                "gbps": round(nbytes / t8 / 1e9, 1), "pct_hbm_peak": round(100 * nbytes / t8 / 1e9 / HBM_PEAK_GBPS, 1),
+                "speedup_vs_dense_fp16": round(dense_us / (t8 * 1e6), 3) if dense_us else None,
+            })
+            log("int8:", int8_cases[-1])
+
     # ---- the compressor: whole compress() call (count pass, read-back of the total, fill pass) -----
     compress_cases = []
     if not args.no_compress:
@@ -396,6 +423,7 @@ def main():
         "cpu_baseline": cpu,
         "cases": per_case,
         "compress": compress_cases,
+        "int8_values_variant": int8_cases,
         "device": dev.name,
     }
     print(json.dumps(out), flush=True)
