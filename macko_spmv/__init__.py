@@ -4,8 +4,11 @@ from macko_spmv_amd import (  # noqa: F401
     LIB_NAME,
     __version__,
     compress,
+    compress_int8,
     decompress,
     move_to_device,
     multiply,
     multiply_axpby,
+    multiply_int8,
+    multiply_int8_axpby,
 )
