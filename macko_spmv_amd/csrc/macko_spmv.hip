@@ -244,17 +244,12 @@ __device__ __forceinline__ void xpiece_issue(u32 byte_offset, const u32x4 &buffe
         asm volatile("buffer_load_dwordx4 v[84:87], %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer)
                      : "memory", "v84", "v85", "v86", "v87");
 }
+// waits for piece j and writes it to LDS straight from its registers
 template <int J, int N>
-__device__ __forceinline__ u32x4 xpiece_take()
+__device__ __forceinline__ void xpiece_to_lds(u32 lds_byte_address)
 {
-    u32x4 v;
-    if (J == 0)
-        asm volatile("s_waitcnt vmcnt(%4)\n\tv_mov_b32 %0, v80\n\tv_mov_b32 %1, v81\n\tv_mov_b32 %2, v82\n\tv_mov_b32 %3, v83"
-                     : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w) : "n"(N) : "memory");
-    if (J == 1)
-        asm volatile("s_waitcnt vmcnt(%4)\n\tv_mov_b32 %0, v84\n\tv_mov_b32 %1, v85\n\tv_mov_b32 %2, v86\n\tv_mov_b32 %3, v87"
-                     : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w) : "n"(N) : "memory");
-    return v;
+    if (J == 0) asm volatile("s_waitcnt vmcnt(%1)\n\tds_write_b128 %0, v[80:83]" ::"v"(lds_byte_address), "n"(N) : "memory");
+    if (J == 1) asm volatile("s_waitcnt vmcnt(%1)\n\tds_write_b128 %0, v[84:87]" ::"v"(lds_byte_address), "n"(N) : "memory");
 }
 
 // ring slot J of a D-deep ring: issue both loads / wait and copy out
@@ -423,33 +418,7 @@ spmv_stream_kernel(const SpmvArgs a)
     int window[2];
     window[0] = probe_take<0, kXLoads + 1>();
     window[1] = probe_take<1, kXLoads>();
-    int range[2];
-    wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
-    // Cut at the row start NEAREST to the target rather than the first one at or after it: with
-    // rows of similar length every wave then gets the same number of rows.
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        const int rr = range[k];
-        if (rr > 0 && rr <= a.rows) {
-            int after, before;
-            if (__builtin_expect(rr - 1 >= base[k] && rr <= base[k] + 63, 1)) {
-                after = __builtin_amdgcn_readlane(window[k], rr - base[k]);
-                before = __builtin_amdgcn_readlane(window[k], rr - 1 - base[k]);
-            } else {
-                after = uniform(a.row_ptr[rr]);
-                before = uniform(a.row_ptr[rr - 1]);
-            }
-            if (target[k] - before < after - target[k]) range[k] = rr - 1;
-        }
-    }
-    if (gw == 0) range[0] = 0;
-    if (gw == n_waves - 1) range[1] = a.rows;
-    const int row_first = uniform(range[0]);
-    const int row_last = uniform(range[1]);
-    MACKO_STAMP(2);
-
-    // ---- 4. my first row and my tile range --------------------------------------------------------------
-    // window of row_ptr values: lane i holds row_ptr[win_base + i]
+    // window of row_ptr values the row loop reads row starts from: lane i holds row_ptr[win_base + i]
     int win_base = base[0];
     int win = window[0];
     auto row_start = [&](int r) -> int {  // r in [win_base, win_base + 63]
@@ -469,34 +438,86 @@ spmv_stream_kernel(const SpmvArgs a)
         }
     };
 
-    // current row r = first non-empty owned row; empty ones are written on the way
-    bool have_work = row_first < row_last;
-    int r = row_first;
+    int row_last = 0;
+    bool have_work = false;
+    int r = 0;  // current row
     int e0 = 0, e1 = 0, s_end = 0;
-    u32 first_tile = 0, last_tile = 0;
-    if (__builtin_expect(have_work, 1)) {
-        slide_window(r);
-        e0 = row_start(r);
-        e1 = row_start(r + 1);
-        while (__builtin_expect(e1 == e0, 0)) {
-            store_row(r, 0.f);
-            ++r;
-            if (r >= row_last) {
-                have_work = false;
-                break;
+    bool resolved = false;
+    {
+        // Straight-line case: both cuts fall inside their probe windows and my first row is not
+        // empty.  Cut k is the first row start at or after target k, or the one before it if that
+        // is nearer (with rows of similar length every wave then gets the same number of rows).
+        const unsigned long long m0 = __ballot(window[0] >= target[0]);
+        const unsigned long long m1 = __ballot(window[1] >= target[1]);
+        const int f0 = m0 ? __builtin_ctzll(m0) : 0;
+        const int f1 = m1 ? __builtin_ctzll(m1) : 0;
+        if (__builtin_expect(f0 >= 1 && f0 <= 62 && f1 >= 1 && gw != n_waves - 1, 1)) {
+            const int at0 = __builtin_amdgcn_readlane(window[0], f0);
+            const int before0 = __builtin_amdgcn_readlane(window[0], f0 - 1);
+            const int at1 = __builtin_amdgcn_readlane(window[1], f1);
+            const int before1 = __builtin_amdgcn_readlane(window[1], f1 - 1);
+            const int back0 = target[0] - before0 < at0 - target[0] ? 1 : 0;
+            const int back1 = target[1] - before1 < at1 - target[1] ? 1 : 0;
+            r = base[0] + f0 - back0;
+            row_last = base[1] + f1 - back1;
+            e0 = back0 ? before0 : at0;
+            e1 = __builtin_amdgcn_readlane(window[0], f0 - back0 + 1);
+            s_end = back1 ? before1 : at1;
+            have_work = r < row_last;
+            resolved = have_work && e1 != e0;
+        }
+    }
+    MACKO_STAMP(2);
+    if (__builtin_expect(!resolved, 0)) {
+        // General case: search rounds where a window missed, first / last wave, leading empty rows.
+        int range[2];
+        wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int rr = range[k];
+            if (rr > 0 && rr <= a.rows) {
+                int after, before;
+                if (rr - 1 >= base[k] && rr <= base[k] + 63) {
+                    after = __builtin_amdgcn_readlane(window[k], rr - base[k]);
+                    before = __builtin_amdgcn_readlane(window[k], rr - 1 - base[k]);
+                } else {
+                    after = uniform(a.row_ptr[rr]);
+                    before = uniform(a.row_ptr[rr - 1]);
+                }
+                if (target[k] - before < after - target[k]) range[k] = rr - 1;
             }
+        }
+        if (gw == 0) range[0] = 0;
+        if (gw == n_waves - 1) range[1] = a.rows;
+        r = uniform(range[0]);
+        row_last = uniform(range[1]);
+        have_work = r < row_last;
+        if (have_work) {  // first non-empty owned row; empty ones are written on the way
             slide_window(r);
             e0 = row_start(r);
             e1 = row_start(r + 1);
+            while (e1 == e0) {
+                store_row(r, 0.f);
+                ++r;
+                if (r >= row_last) {
+                    have_work = false;
+                    break;
+                }
+                slide_window(r);
+                e0 = row_start(r);
+                e1 = row_start(r + 1);
+            }
         }
+        if (have_work)  // end of my last owned row
+            s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
     }
+
+    // ---- 4. my tile range; the ring is filled with my first D tiles before x is even in LDS: they
+    //         fly while the workgroup finishes the copy and meets at the barrier -------------------------
+    u32 first_tile = 0, last_tile = 0;
     if (__builtin_expect(have_work, 1)) {
-        // end of my last owned row
-        s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
         first_tile = (u32)e0 >> kTileShift;
         last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
-        // Fill the ring with my first D tiles before x is even in LDS: they fly while the
-        // workgroup finishes the copy and meets at the barrier.
         static_for<D>([&](auto slot) {
             constexpr int J = decltype(slot)::value;
             issue_slot(slot, first_tile + J, first_tile + J < last_tile);
@@ -505,17 +526,17 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 5. x pieces into LDS (older than the ring loads just issued, if any) ---------------------------
     if (X_LDS) {
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(lds + kLdsFront);
-        u32x4 x0, x1;
+        const u32 lds_x = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
+        const u32 dst0 = lds_x + (u32)tid * 16, dst1 = dst0 + BLOCK * 16;
         if (__builtin_expect(have_work, 1)) {
-            x0 = xpiece_take<0, kTileLoads + 1>();
-            x1 = xpiece_take<1, kTileLoads>();
+            if (tid < x_nvec) xpiece_to_lds<0, kTileLoads + 1>(dst0);
+            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, kTileLoads>(dst1);
         } else {
-            x0 = xpiece_take<0, 1>();
-            x1 = xpiece_take<1, 0>();
+            if (tid < x_nvec) xpiece_to_lds<0, 1>(dst0);
+            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, 0>(dst1);
         }
-        if (tid < x_nvec) d4[tid] = x0;
-        if (tid + BLOCK < x_nvec) d4[tid + BLOCK] = x1;
+        // the copies above are asm the compiler's wait tracking does not see
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         MACKO_STAMP(3);
         __syncthreads();
     }
