@@ -359,7 +359,12 @@ spmv_stream_kernel(const SpmvArgs a)
     const int lane = tid & (kWave - 1);
     const int wave = uniform(tid >> 6);
     const u32 n_waves = gridDim.x * WAVES;
-    const u32 gw = blockIdx.x * WAVES + wave;
+    // Workgroups are dealt round-robin to the 8 XCDs (workgroup i runs on XCD i % 8).  Giving XCD k
+    // the k-th contiguous eighth of the matrix keeps neighbouring workgroups, which share boundary
+    // tiles, behind one L2.
+    u32 wg = blockIdx.x;
+    if ((gridDim.x & 7) == 0) wg = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const u32 gw = wg * WAVES + wave;
     MACKO_STAMP(0);
 
 
