@@ -46,6 +46,10 @@ struct SpmvArgs {
     // w*rows_q + ((w*rows_frac) >> 32) with rows_frac = floor((rows % W) * 2^32 / W).
     u32 entries_q, entries_rem;
     u32 rows_q, rows_frac;
+    // 1 when there are no more rows than waves: wave w then simply owns rows
+    // [floor(w*rows/W), floor((w+1)*rows/W)), at most one row each.  No split of whole rows can do
+    // better than the longest row, and cutting by entries could hand one wave two rows.
+    u32 row_even;
 #ifdef MACKO_SPMV_TRACE
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif
@@ -381,12 +385,14 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 1. tracked loads, oldest first: row_ptr probes, x pieces ------------------------------------
     // probes: 64 consecutive row_ptr values around where my first / last row should be
-    int target[2], base[2];
+    int target[2], base[2], guess[2];
     {
         target[0] = (int)even_split(gw, a.entries_q, a.entries_rem);  // < P < 2^31
         target[1] = (int)even_split(gw + 1, a.entries_q, a.entries_rem);
-        base[0] = probe_base((int)(gw * a.rows_q + __umulhi(gw, a.rows_frac)), a.rows);
-        base[1] = probe_base((int)((gw + 1) * a.rows_q + __umulhi(gw + 1, a.rows_frac)), a.rows);
+        guess[0] = (int)(gw * a.rows_q + __umulhi(gw, a.rows_frac));
+        guess[1] = gw == n_waves - 1 ? a.rows : (int)((gw + 1) * a.rows_q + __umulhi(gw + 1, a.rows_frac));
+        base[0] = probe_base(guess[0], a.rows);
+        base[1] = probe_base(guess[1], a.rows);
         int i0 = base[0] + lane, i1 = base[1] + lane;
         i0 = i0 <= a.rows ? i0 : a.rows;
         i1 = i1 <= a.rows ? i1 : a.rows;
@@ -456,7 +462,17 @@ spmv_stream_kernel(const SpmvArgs a)
         const unsigned long long m1 = __ballot(window[1] >= target[1]);
         const int f0 = m0 ? __builtin_ctzll(m0) : 0;
         const int f1 = m1 ? __builtin_ctzll(m1) : 0;
-        if (__builtin_expect(f0 >= 1 && f0 <= 62 && f1 >= 1 && gw != n_waves - 1, 1)) {
+        if (a.row_even) {  // the cuts are the guesses themselves; both lie inside their windows
+            r = guess[0];
+            row_last = guess[1];
+            have_work = r < row_last;
+            if (have_work) {  // then r <= rows - 1 and r + 1 - base[0] <= 63
+                e0 = __builtin_amdgcn_readlane(window[0], r - base[0]);
+                e1 = __builtin_amdgcn_readlane(window[0], r + 1 - base[0]);
+                s_end = __builtin_amdgcn_readlane(window[1], row_last - base[1]);
+            }
+            resolved = have_work && e1 != e0;
+        } else if (__builtin_expect(f0 >= 1 && f0 <= 62 && f1 >= 1 && gw != n_waves - 1, 1)) {
             const int at0 = __builtin_amdgcn_readlane(window[0], f0);
             const int before0 = __builtin_amdgcn_readlane(window[0], f0 - 1);
             const int at1 = __builtin_amdgcn_readlane(window[1], f1);
@@ -475,10 +491,10 @@ spmv_stream_kernel(const SpmvArgs a)
     MACKO_STAMP(2);
     if (__builtin_expect(!resolved, 0)) {
         // General case: search rounds where a window missed, first / last wave, leading empty rows.
-        int range[2];
-        wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
+        int range[2] = {guess[0], guess[1]};
+        if (!a.row_even) wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
+        for (int k = 0; k < 2 && !a.row_even; ++k) {
             const int rr = range[k];
             if (rr > 0 && rr <= a.rows) {
                 int after, before;
@@ -698,6 +714,7 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
     a.entries_rem = (u32)(a.padded % n_waves);
     a.rows_q = (u32)a.rows / n_waves;
     a.rows_frac = (u32)(((unsigned long long)((u32)a.rows % n_waves) << 32) / n_waves);
+    a.row_even = (u32)a.rows <= n_waves ? 1u : 0u;
     if (lds_bytes > 64 * 1024) {
         // one-time opt-in to more than 64 KiB of dynamic LDS, per device
         static bool done[64] = {};
@@ -814,7 +831,7 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
-               0,                   0,                   0,              0};
+               0,                   0,                   0,              0,             0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = g_trace;
 #endif
@@ -830,7 +847,7 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
-               0,                   0,                   0,              0};
+               0,                   0,                   0,              0,             0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
@@ -846,7 +863,7 @@ extern "C" int macko_spmv_i8f16(const void *values, const void *deltas, const in
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
-               0,                   0,                   0,              0};
+               0,                   0,                   0,              0,             0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
@@ -862,7 +879,7 @@ extern "C" int macko_spmv_i8f16_axpby(const void *values, const void *deltas, co
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
-               0,                   0,                   0,              0};
+               0,                   0,                   0,              0,             0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
