@@ -302,6 +302,22 @@ def main():
     # ---- per-case timing, MACKO and dense, each over >= 1 GB of distinct copies ------------------
     per_case = []
     if not args.no_dense:
+        import ctypes
+
+        hip = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
+        hip.macko_calibration_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+        read_pool = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+        read_sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+        def read_launches(nbytes):
+            # pure streaming read of the same number of bytes, rotating through 1 GiB
+            nbytes = int(nbytes) // 16 * 16
+            stride = (nbytes + 4095) // 4096 * 4096
+            sp = torch.cuda.current_stream().cuda_stream
+            for k in range(max(2, (1 << 30) // stride)):
+                rc = hip.macko_calibration_read(read_pool.data_ptr() + k * stride, nbytes, read_sink.data_ptr(), sp)
+                assert rc == 0, rc
+
         for c in cases:
             n_sparse = max(2, min(256, int(1.0e9 // c["bytes"]) + 1))
             copies = c["copies"] + [clone_compressed(c["copies"][0]) for _ in range(n_sparse - 2)]
@@ -315,6 +331,8 @@ def main():
                                     args.case_replays)
             t_dense /= len(dense_copies)
             del dense_copies
+            t_read, _ = time_graph(torch, lambda: read_launches(c["bytes"]), args.case_replays)
+            t_read /= max(2, (1 << 30) // ((int(c["bytes"]) // 16 * 16 + 4095) // 4096 * 4096))
             per_case.append({
                 "shape": f"{c['rows']}x{c['cols']}", "density": c["density"],
                 "macko_us": round(t_sparse * 1e6, 2), "dense_us": round(t_dense * 1e6, 2),
@@ -322,6 +340,7 @@ def main():
                 "macko_gbps": round(c["bytes"] / t_sparse / 1e9, 1),
                 "pct_hbm_peak": round(100 * c["bytes"] / t_sparse / 1e9 / HBM_PEAK_GBPS, 1),
                 "dense_gbps": round(db / t_dense / 1e9, 1),
+                "stream_read_us": round(t_read * 1e6, 2),
             })
             log(per_case[-1])
 
@@ -388,6 +407,17 @@ def main():
         v = [p["speedup_vs_dense"] for p in per_case if p["density"] == d]
         return round(sum(v) / len(v), 3) if v else None
 
+    yardstick = None
+    if per_case:
+        t_m = sum(p["macko_us"] for p in per_case)
+        t_r = sum(p["stream_read_us"] for p in per_case)
+        yardstick = {
+            "what": "calibration_read_kernel: one launch that only reads the same number of bytes (256x1024 "
+                    "threads, contiguous span per wave), timed like the per-case SpMV figures",
+            "us_per_launch": round(t_r / len(per_case), 3),
+            "gbps": round(step_bytes / t_r / 1e3, 1),
+            "spmv_time_over_read_time": round(t_m / t_r, 3),
+        }
     bytes_per_launch = step_bytes / n_launch
     out = {
         "metric": "SpMV effective HBM GB/s (% of ~8 TB/s) + speedup vs dense fp16 GEMV",
@@ -421,6 +451,7 @@ def main():
             "us_per_launch": round(launch_us, 3),
         },
         "cpu_baseline": cpu,
+        "streaming_read_yardstick": yardstick,
         "cases": per_case,
         "compress": compress_cases,
         "int8_values_variant": int8_cases,
