@@ -25,7 +25,7 @@ HIP_LIB = "libmacko_hip.so"
 TORCH_LIB = "libmacko_torch.so"
 ARCH = "gfx950"
 
-HIP_SOURCES = ["macko_spmv.hip", "macko_compress.hip", "macko_runtime.hip"]
+HIP_SOURCES = ["macko_spmv.hip", "macko_compress.hip", "macko_runtime.hip", "macko_decode.hip"]
 TORCH_SOURCES = ["macko_torch.cpp"]
 
 

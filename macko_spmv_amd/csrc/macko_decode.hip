@@ -1,0 +1,206 @@
+// Glue kernels of the batch-1 decode harness (gfx950, wave64): everything a Llama-architecture
+// decode step does between the projections, one launch each, so that the step is dominated by the
+// matrix-vector products it is there to measure.  The upstream harness runs stock Hugging Face
+// modules for these parts (python_scripts/util_run_pruned_llm.py:136-160); there is no upstream
+// kernel to mirror.  All activations are fp16, all arithmetic fp32.  The current position is read
+// from device memory so a captured HIP graph can be replayed for every token.
+
+#include "macko_common.h"
+#include "macko_decode.h"
+
+namespace macko {
+namespace {
+
+__device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+
+// Sum over the workgroup (blockDim.x a multiple of 64, at most 1024); every thread gets the total.
+__device__ __forceinline__ float block_sum(float v, float *scratch /* [17] */)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const float w = wave_sum(v);
+    __syncthreads();  // scratch may still be read from an earlier call
+    if (lane == 0) scratch[wave] = w;
+    __syncthreads();
+    float total = 0.f;
+    for (int i = 0; i < n_waves; ++i) total += scratch[i];
+    return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float *scratch)
+{
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    float m = v;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    __syncthreads();
+    if (lane == 0) scratch[wave] = m;
+    __syncthreads();
+    float total = scratch[0];
+    for (int i = 1; i < n_waves; ++i) total = fmaxf(total, scratch[i]);
+    return total;
+}
+
+// y = x * rsqrt(mean(x^2) + eps) * w, one workgroup.
+__global__ void __launch_bounds__(1024) rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
+                                                       uint16_t *__restrict__ y, int n, float eps)
+{
+    __shared__ float scratch[17];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = h2f(x[i]);
+        ss += v * v;
+    }
+    const float inv = rsqrtf(block_sum(ss, scratch) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += blockDim.x) y[i] = f2h(h2f(x[i]) * inv * h2f(w[i]));
+}
+
+// Rotary embedding of q and k (rotate-half convention: element i pairs with i + head_dim/2), k and
+// v appended to the caches at the current position.  One workgroup per head, head_dim/2 threads.
+// q, k, v: [n_heads * head_dim]; cos, sin: [max_len, head_dim/2] fp32; caches [n_heads, max_len, head_dim].
+__global__ void rope_append_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
+                                   const uint16_t *__restrict__ v, const float *__restrict__ cos_table,
+                                   const float *__restrict__ sin_table, const long long *__restrict__ position,
+                                   uint16_t *__restrict__ q_out, uint16_t *__restrict__ k_cache,
+                                   uint16_t *__restrict__ v_cache, int head_dim, int max_len)
+{
+    const int head = blockIdx.x, i = threadIdx.x, half = head_dim >> 1;
+    long long pos = position[0];
+    pos = pos < 0 ? 0 : (pos >= max_len ? max_len - 1 : pos);
+    const float c = cos_table[pos * half + i], s = sin_table[pos * half + i];
+    const size_t in = (size_t)head * head_dim;
+    const size_t slot = ((size_t)head * max_len + (size_t)pos) * head_dim;
+    const float q0 = h2f(q[in + i]), q1 = h2f(q[in + i + half]);
+    q_out[in + i] = f2h(q0 * c - q1 * s);
+    q_out[in + i + half] = f2h(q1 * c + q0 * s);
+    const float k0 = h2f(k[in + i]), k1 = h2f(k[in + i + half]);
+    k_cache[slot + i] = f2h(k0 * c - k1 * s);
+    k_cache[slot + i + half] = f2h(k1 * c + k0 * s);
+    v_cache[slot + i] = v[in + i];
+    v_cache[slot + i + half] = v[in + i + half];
+}
+
+// Single-query attention over positions 0..position of one head per workgroup (256 threads):
+// scores, softmax, weighted sum of v.  head_dim <= 256 and a multiple of 8; max_len <= kMaxLen.
+constexpr int kAttnThreads = 256;
+constexpr int kMaxLen = 4096;
+__global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t *__restrict__ q,
+                                                                  const uint16_t *__restrict__ k_cache,
+                                                                  const uint16_t *__restrict__ v_cache,
+                                                                  const long long *__restrict__ position,
+                                                                  uint16_t *__restrict__ out, int head_dim, int max_len,
+                                                                  float scale)
+{
+    __shared__ float scores[kMaxLen];
+    __shared__ float qs[256];
+    __shared__ float partial[kAttnThreads];
+    __shared__ float scratch[17];
+    const int head = blockIdx.x, tid = threadIdx.x;
+    long long pos = position[0];
+    pos = pos < 0 ? 0 : (pos >= max_len ? max_len - 1 : pos);
+    const int len = (int)pos + 1;
+    if (tid < head_dim) qs[tid] = h2f(q[(size_t)head * head_dim + tid]) * scale;
+    __syncthreads();
+    const uint16_t *kh = k_cache + (size_t)head * max_len * head_dim;
+    const uint16_t *vh = v_cache + (size_t)head * max_len * head_dim;
+    float local_max = -3.0e38f;
+    for (int p = tid; p < len; p += kAttnThreads) {
+        const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)p * head_dim);
+        float acc = 0.f;
+        for (int j = 0; j < head_dim / 8; ++j) {
+            const u32x4 kv = row[j];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc += h2f((uint16_t)(kv[e] & 0xffffu)) * qs[8 * j + 2 * e];
+                acc += h2f((uint16_t)(kv[e] >> 16)) * qs[8 * j + 2 * e + 1];
+            }
+        }
+        scores[p] = acc;
+        local_max = fmaxf(local_max, acc);
+    }
+    const float m = block_max(local_max, scratch);
+    float local_sum = 0.f;
+    for (int p = tid; p < len; p += kAttnThreads) {
+        const float e = __expf(scores[p] - m);
+        scores[p] = e;
+        local_sum += e;
+    }
+    const float inv = 1.0f / block_sum(local_sum, scratch);  // also orders the scores[] writes
+    // thread (g, d): dims d = tid % head_dim, position slices g = tid / head_dim
+    const int groups = kAttnThreads / head_dim > 0 ? kAttnThreads / head_dim : 1;
+    const int d = tid % head_dim, g = tid / head_dim;
+    float acc = 0.f;
+    if (g < groups)
+        for (int p = g; p < len; p += groups) acc += scores[p] * h2f(vh[(size_t)p * head_dim + d]);
+    partial[tid] = acc;
+    __syncthreads();
+    if (tid < head_dim) {
+        float total = 0.f;
+        for (int gg = 0; gg < groups; ++gg) total += partial[gg * head_dim + tid];
+        out[(size_t)head * head_dim + tid] = f2h(total * inv);
+    }
+}
+
+// out[i] = silu(gate[i]) * up[i]
+__global__ void silu_mul_kernel(const uint16_t *__restrict__ gate, const uint16_t *__restrict__ up,
+                                uint16_t *__restrict__ out, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float gv = h2f(gate[i]);
+        out[i] = f2h(gv / (1.0f + __expf(-gv)) * h2f(up[i]));
+    }
+}
+
+}  // namespace
+}  // namespace macko
+
+extern "C" int macko_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int32_t n, float eps, void *stream)
+{
+    using namespace macko;
+    if (x == nullptr || weight == nullptr || y == nullptr || n <= 0) return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(1024), 0, as_stream(stream), (const uint16_t *)x,
+                       (const uint16_t *)weight, (uint16_t *)y, n, eps);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_decode_rope_append_f16(const void *q, const void *k, const void *v, const float *cos_table,
+                                            const float *sin_table, const int64_t *position, void *q_out,
+                                            void *k_cache, void *v_cache, int32_t n_heads, int32_t head_dim,
+                                            int32_t max_len, void *stream)
+{
+    using namespace macko;
+    if (!q || !k || !v || !cos_table || !sin_table || !position || !q_out || !k_cache || !v_cache)
+        return MACKO_E_INVALID_ARGUMENT;
+    if (n_heads <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 2048 || max_len <= 0)
+        return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(rope_append_kernel, dim3(n_heads), dim3(head_dim / 2), 0, as_stream(stream),
+                       (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, cos_table, sin_table,
+                       (const long long *)position, (uint16_t *)q_out, (uint16_t *)k_cache, (uint16_t *)v_cache,
+                       head_dim, max_len);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache,
+                                          const int64_t *position, void *out, int32_t n_heads, int32_t head_dim,
+                                          int32_t max_len, float scale, void *stream)
+{
+    using namespace macko;
+    if (!q || !k_cache || !v_cache || !position || !out) return MACKO_E_INVALID_ARGUMENT;
+    if (n_heads <= 0 || head_dim <= 0 || head_dim > 256 || (head_dim & 7) || max_len <= 0 || max_len > kMaxLen)
+        return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(k_cache) & 15)) return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(attention_kernel, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
+                       (const uint16_t *)q, (const uint16_t *)k_cache, (const uint16_t *)v_cache,
+                       (const long long *)position, (uint16_t *)out, head_dim, max_len, scale);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_decode_silu_mul_f16(const void *gate, const void *up, void *out, int32_t n, void *stream)
+{
+    using namespace macko;
+    if (!gate || !up || !out || n <= 0) return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((n + 255) / 256), dim3(256), 0, as_stream(stream),
+                       (const uint16_t *)gate, (const uint16_t *)up, (uint16_t *)out, n);
+    return (int)hipGetLastError();
+}

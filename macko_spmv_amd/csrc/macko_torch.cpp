@@ -16,6 +16,7 @@
 
 #include <tuple>
 
+#include "macko_decode.h"
 #include "macko_hip.h"
 
 namespace {
@@ -210,6 +211,90 @@ at::Tensor decompress_hip(const at::Tensor &M_values, const at::Tensor &M_deltas
     return dense;
 }
 
+// ---- glue kernels of the decode harness (include/macko_decode.h) -------------------------------
+
+void check_half_gpu(const at::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.is_cuda() && t.dtype() == at::kHalf && t.is_contiguous(), name,
+                " must be a contiguous torch.half GPU tensor");
+}
+
+at::Tensor decode_rmsnorm_hip(const at::Tensor &x, const at::Tensor &weight, double eps)
+{
+    check_half_gpu(x, "x");
+    check_half_gpu(weight, "weight");
+    TORCH_CHECK(weight.numel() == x.numel(), "weight and x must have the same length");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    at::Tensor y = at::empty_like(x);
+    check_rc(macko_decode_rmsnorm_f16(x.data_ptr(), weight.data_ptr(), y.data_ptr(), (int32_t)x.numel(), (float)eps,
+                                      (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "decode_rmsnorm");
+    return y;
+}
+
+// q, k, v: [n_heads * head_dim]; caches [n_heads, max_len, head_dim] (updated in place); returns rotated q.
+at::Tensor decode_rope_append_hip(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
+                                  const at::Tensor &cos_table, const at::Tensor &sin_table,
+                                  const at::Tensor &position, at::Tensor k_cache, at::Tensor v_cache)
+{
+    check_half_gpu(q, "q");
+    check_half_gpu(k, "k");
+    check_half_gpu(v, "v");
+    check_half_gpu(k_cache, "k_cache");
+    check_half_gpu(v_cache, "v_cache");
+    TORCH_CHECK(k_cache.dim() == 3 && v_cache.sizes() == k_cache.sizes(), "caches must be [heads, max_len, head_dim]");
+    const int64_t n_heads = k_cache.size(0), max_len = k_cache.size(1), head_dim = k_cache.size(2);
+    TORCH_CHECK(q.numel() == n_heads * head_dim && k.numel() == q.numel() && v.numel() == q.numel(), "bad q/k/v size");
+    TORCH_CHECK(cos_table.is_cuda() && cos_table.dtype() == at::kFloat && cos_table.is_contiguous() &&
+                    cos_table.numel() == max_len * (head_dim / 2) && sin_table.is_cuda() &&
+                    sin_table.dtype() == at::kFloat && sin_table.is_contiguous() &&
+                    sin_table.numel() == cos_table.numel(),
+                "cos/sin tables must be contiguous float32 GPU tensors [max_len, head_dim/2]");
+    TORCH_CHECK(position.is_cuda() && position.dtype() == at::kLong && position.numel() == 1, "bad position");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    at::Tensor q_out = at::empty_like(q);
+    check_rc(macko_decode_rope_append_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_table.data_ptr<float>(),
+                                          sin_table.data_ptr<float>(), position.data_ptr<int64_t>(), q_out.data_ptr(),
+                                          k_cache.data_ptr(), v_cache.data_ptr(), (int32_t)n_heads, (int32_t)head_dim,
+                                          (int32_t)max_len,
+                                          (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "decode_rope_append");
+    return q_out;
+}
+
+at::Tensor decode_attention_hip(const at::Tensor &q, const at::Tensor &k_cache, const at::Tensor &v_cache,
+                                const at::Tensor &position, double scale)
+{
+    check_half_gpu(q, "q");
+    check_half_gpu(k_cache, "k_cache");
+    check_half_gpu(v_cache, "v_cache");
+    TORCH_CHECK(k_cache.dim() == 3 && v_cache.sizes() == k_cache.sizes(), "caches must be [heads, max_len, head_dim]");
+    const int64_t n_heads = k_cache.size(0), max_len = k_cache.size(1), head_dim = k_cache.size(2);
+    TORCH_CHECK(q.numel() == n_heads * head_dim, "bad q size");
+    TORCH_CHECK(position.is_cuda() && position.dtype() == at::kLong && position.numel() == 1, "bad position");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    at::Tensor out = at::empty_like(q);
+    check_rc(macko_decode_attention_f16(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                        position.data_ptr<int64_t>(), out.data_ptr(), (int32_t)n_heads,
+                                        (int32_t)head_dim, (int32_t)max_len, (float)scale,
+                                        (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "decode_attention");
+    return out;
+}
+
+at::Tensor decode_silu_mul_hip(const at::Tensor &gate, const at::Tensor &up)
+{
+    check_half_gpu(gate, "gate");
+    check_half_gpu(up, "up");
+    TORCH_CHECK(gate.numel() == up.numel(), "gate and up must have the same length");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(gate.device());
+    at::Tensor out = at::empty_like(gate);
+    check_rc(macko_decode_silu_mul_f16(gate.data_ptr(), up.data_ptr(), out.data_ptr(), (int32_t)gate.numel(),
+                                       (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "decode_silu_mul");
+    return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(macko_spmv, m)
@@ -224,6 +309,11 @@ TORCH_LIBRARY(macko_spmv, m)
           "Tensor V) -> Tensor");
     m.def("multiply_int8_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
           "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
+    m.def("decode_rmsnorm(Tensor x, Tensor weight, float eps) -> Tensor");
+    m.def("decode_rope_append(Tensor q, Tensor k, Tensor v, Tensor cos_table, Tensor sin_table, Tensor position, "
+          "Tensor(a!) k_cache, Tensor(b!) v_cache) -> Tensor");
+    m.def("decode_attention(Tensor q, Tensor k_cache, Tensor v_cache, Tensor position, float scale) -> Tensor");
+    m.def("decode_silu_mul(Tensor gate, Tensor up) -> Tensor");
     m.def("decompress(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols) -> Tensor");
 }
 
@@ -235,6 +325,10 @@ TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
     m.impl("compress_int8", &compress_int8_hip);
     m.impl("multiply_int8", &multiply_int8_hip);
     m.impl("multiply_int8_axpby", &multiply_int8_axpby_hip);
+    m.impl("decode_rmsnorm", &decode_rmsnorm_hip);
+    m.impl("decode_rope_append", &decode_rope_append_hip);
+    m.impl("decode_attention", &decode_attention_hip);
+    m.impl("decode_silu_mul", &decode_silu_mul_hip);
     m.impl("decompress", &decompress_hip);
 }
 

@@ -245,6 +245,162 @@ def greedy_decode(model, prompt, new_tokens, use_graph=True):
     return out, time.perf_counter() - start
 
 
+# ---- a lean single-token decode step ----------------------------------------------------------------
+
+def concat_compressed(parts):
+    """Stack compressed matrices with equal column counts row-wise.  The result is bit-identical to
+    compressing the row-wise concatenation of the dense matrices (rows are compressed independently;
+    only the nibble stream has to be re-packed when a part holds an odd number of entries)."""
+    cols = parts[0][4]
+    assert all(p[4] == cols for p in parts)
+    values, nibbles, row_ptrs, base, rows = [], [], [parts[0][2].new_zeros(1)], 0, 0
+    for v, d, rp, r, _ in parts:
+        n = int(rp[-1].item())
+        values.append(v[:n])
+        nibbles.append(torch.stack((d & 15, d >> 4), dim=1).reshape(-1)[:n])
+        row_ptrs.append(rp[1:] + base)
+        base += n
+        rows += r
+    pad = (-base) % 8
+    values = torch.cat(values + [values[0].new_zeros(pad)])
+    nib = torch.cat(nibbles + [nibbles[0].new_zeros(pad)]).view(-1, 2)
+    deltas = (nib[:, 0] | (nib[:, 1] << 4)).contiguous()
+    return values.contiguous(), deltas, torch.cat(row_ptrs).contiguous(), rows, cols
+
+
+class DecodeEngine:
+    """One token in, logits out, with as few launches as the architecture allows: q|k|v and gate|up
+    stacked into one matrix each, residual additions folded into the o_proj / down_proj products
+    (y = Mx + y), and the parts between the products (RMSNorm, rotary + KV-cache append, attention,
+    SiLU * up) as one hand-written kernel each.  Works on a LlamaDecoder whose projections are either
+    nn.Linear (dense) or MackoLinear; the model's projection modules are consumed (set to None) so
+    the weights are held once."""
+
+    def __init__(self, model):
+        ops = torch.ops.macko_spmv
+        self.ops = ops
+        body = model.model
+        first = body.layers[0].self_attn
+        self.n_heads, self.head_dim, self.max_len = first.n_heads, first.head_dim, first.max_len
+        self.scale = 1.0 / math.sqrt(self.head_dim)
+        dev = body.embed_tokens.weight.device
+        half = self.head_dim // 2
+        inv = 1.0 / (10000.0 ** (torch.arange(0, self.head_dim, 2, device=dev).float() / self.head_dim))
+        ang = torch.outer(torch.arange(self.max_len, device=dev).float(), inv)
+        assert ang.shape == (self.max_len, half)
+        self.cos, self.sin = ang.cos().contiguous(), ang.sin().contiguous()
+        self.embed = body.embed_tokens.weight.data
+        self.final_norm = body.norm.weight.data.contiguous()
+        self.eps = body.norm.eps
+        self.lm_head = model.lm_head.weight.data
+        self.layers = []
+        for layer in body.layers:
+            att, mlp = layer.self_attn, layer.mlp
+            entry = {
+                "norm1": layer.input_layernorm.weight.data.contiguous(),
+                "norm2": layer.post_attention_layernorm.weight.data.contiguous(),
+                "qkv": self._fuse([att.q_proj, att.k_proj, att.v_proj]),
+                "o": self._fuse([att.o_proj]),
+                "gate_up": self._fuse([mlp.gate_proj, mlp.up_proj]),
+                "down": self._fuse([mlp.down_proj]),
+                "k_cache": torch.zeros(self.n_heads, self.max_len, self.head_dim, dtype=torch.float16, device=dev),
+                "v_cache": torch.zeros(self.n_heads, self.max_len, self.head_dim, dtype=torch.float16, device=dev),
+            }
+            att.q_proj = att.k_proj = att.v_proj = att.o_proj = None
+            mlp.gate_proj = mlp.up_proj = mlp.down_proj = None
+            att.k_cache = att.v_cache = None
+            self.layers.append(entry)
+        self.dim = self.embed.shape[1]
+        self.hidden = self.layers[0]["gate_up"][3] // 2 if isinstance(self.layers[0]["gate_up"], tuple) \
+            else self.layers[0]["gate_up"].shape[0] // 2
+
+    @staticmethod
+    def _fuse(mods):
+        if isinstance(mods[0], MackoLinear):
+            parts = [(m.c_0, m.c_1, m.c_2, m.c_3, m.c_4) for m in mods]
+            return parts[0] if len(parts) == 1 else concat_compressed(parts)
+        ws = [m.weight.data for m in mods]
+        return ws[0].contiguous() if len(ws) == 1 else torch.cat(ws, dim=0).contiguous()
+
+    @staticmethod
+    def _matvec(W, x):
+        if isinstance(W, tuple):
+            return macko_spmv.multiply(W, x)
+        return torch.mv(W, x)
+
+    @staticmethod
+    def _matvec_add(W, x, residual):
+        """residual += W x, in place."""
+        if isinstance(W, tuple):
+            macko_spmv.multiply_axpby(W, x, residual, 1.0, 1.0)
+        else:
+            residual.addmv_(W, x)
+
+    def weight_bytes(self):
+        total = 0
+        for entry in self.layers:
+            for key in ("qkv", "o", "gate_up", "down"):
+                W = entry[key]
+                total += (W[0].numel() * 2 + W[1].numel() + W[2].numel() * 4) if isinstance(W, tuple) else W.numel() * 2
+        return total
+
+    def step(self, token, position):
+        """token (1,) int64, position (1,) int64, both on the GPU -> logits (vocab,) fp16."""
+        ops, H, I = self.ops, self.dim, self.hidden
+        x = self.embed.index_select(0, token).view(-1)
+        for L in self.layers:
+            h = ops.decode_rmsnorm(x, L["norm1"], self.eps)
+            qkv = self._matvec(L["qkv"], h)
+            q = ops.decode_rope_append(qkv[:H], qkv[H:2 * H], qkv[2 * H:], self.cos, self.sin, position,
+                                       L["k_cache"], L["v_cache"])
+            a = ops.decode_attention(q, L["k_cache"], L["v_cache"], position, self.scale)
+            self._matvec_add(L["o"], a, x)
+            h = ops.decode_rmsnorm(x, L["norm2"], self.eps)
+            gu = self._matvec(L["gate_up"], h)
+            self._matvec_add(L["down"], ops.decode_silu_mul(gu[:I], gu[I:]), x)
+        return torch.mv(self.lm_head, ops.decode_rmsnorm(x, self.final_norm, self.eps))
+
+
+def engine_decode(engine, prompt, new_tokens, use_graph=True):
+    """Feed `prompt` (1, t) token by token, then generate `new_tokens` greedily.  Returns
+    (generated ids (new_tokens,), seconds spent generating)."""
+    device = prompt.device
+    t = prompt.shape[1]
+    token = prompt[0, :1].clone()
+    position = torch.zeros(1, dtype=torch.long, device=device)
+
+    def step():
+        nxt = engine.step(token, position).argmax(-1, keepdim=True)
+        token.copy_(nxt)
+        position.add_(1)
+
+    run = step
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()                                            # warm-up outside capture (position 0)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        run = graph.replay
+    position.zero_()
+    for i in range(t):                                        # prefill: same step, the prediction is discarded
+        token.copy_(prompt[0, i:i + 1])
+        run()
+    out = torch.zeros(new_tokens, dtype=torch.long, device=device)
+    out[0] = token[0]
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for i in range(1, new_tokens):
+        run()
+        out[i] = token[0]
+    torch.cuda.synchronize()
+    return out, time.perf_counter() - start
+
+
 def build_model(density, n_layers, dim, hidden, n_heads, vocab, max_len, seed=0, sparse=True):
     """Random Llama-architecture fp16 model on the GPU with every projection pruned per row to
     `density`; with sparse=True the projections are replaced by MackoLinear.  Returns (model, bytes
@@ -281,16 +437,25 @@ def main(argv=None):
     ap.add_argument("--tokens", type=int, default=256)
     ap.add_argument("--runs", type=int, default=3)
     ap.add_argument("--skip-dense", action="store_true")
+    ap.add_argument("--module-path", action="store_true",
+                    help="decode through the nn.Module forward (one framework kernel per elementary op) "
+                         "instead of the lean DecodeEngine step")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "needs a GPU"
     torch.set_grad_enabled(False)
     max_len = args.prompt + args.tokens + 8
-    result = {"density": args.density, "layers": args.layers, "prompt": args.prompt, "tokens": args.tokens}
+    result = {"density": args.density, "layers": args.layers, "prompt": args.prompt, "tokens": args.tokens,
+              "path": "module" if args.module_path else "engine"}
     for label, sparse in (("dense", False), ("macko", True)):
         if label == "dense" and args.skip_dense:
             continue
         model, proj_bytes = build_model(args.density, args.layers, args.dim, args.hidden, args.heads, args.vocab,
                                         max_len, sparse=sparse)
+        engine = None
+        if not args.module_path:
+            engine = DecodeEngine(model)
+            proj_bytes = engine.weight_bytes()
+            torch.cuda.empty_cache()
         resident = torch.cuda.memory_allocated()
         torch.cuda.reset_peak_memory_stats()  # the peak below covers prefill + decode, not model construction
         g = torch.Generator(device="cuda")
@@ -298,7 +463,10 @@ def main(argv=None):
         prompt = torch.randint(0, args.vocab, (1, args.prompt), device="cuda", generator=g)
         times = []
         for _ in range(args.runs):
-            ids, seconds = greedy_decode(model, prompt, args.tokens)
+            if engine is not None:
+                ids, seconds = engine_decode(engine, prompt, args.tokens)
+            else:
+                ids, seconds = greedy_decode(model, prompt, args.tokens)
             times.append(seconds)
         best = min(times)
         result[label] = {
@@ -309,7 +477,7 @@ def main(argv=None):
             "first_tokens": ids[:8].tolist(),
         }
         print(label, result[label], file=sys.stderr, flush=True)
-        del model
+        del model, engine
         torch.cuda.empty_cache()
     if "dense" in result and "macko" in result:
         result["speedup"] = round(result["macko"]["tokens_per_s"] / result["dense"]["tokens_per_s"], 3)

@@ -12,22 +12,27 @@ import macko_spmv
 import macko_spmv_amd
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "macko_hip.h")
+HEADERS = [os.path.join(ROOT, "include", name) for name in sorted(os.listdir(os.path.join(ROOT, "include")))
+           if name.endswith(".h")]
 
 
 def _declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(macko_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(macko_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_symbols_are_exported():
     names = _declared_symbols()
     assert {"macko_spmv_f16", "macko_spmv_f16_axpby", "macko_compress_f16_count", "macko_compress_f16_fill",
-            "macko_decompress_f16", "macko_hip_error_string", "macko_hip_abi_version"} <= set(names)
+            "macko_decompress_f16", "macko_hip_error_string", "macko_hip_abi_version", "macko_spmv_i8f16",
+            "macko_compress_i8_count", "macko_compress_i8_fill", "macko_decode_attention_f16"} <= set(names)
     lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
     for name in names:
-        assert hasattr(lib, name), f"{name} declared in include/macko_hip.h but not exported"
+        assert hasattr(lib, name), f"{name} declared under include/ but not exported"
 
 
 def test_abi_version_and_error_strings():

@@ -66,3 +66,87 @@ def test_decode_dense_vs_compressed_state_dict_and_graph_replay():
     assert torch.equal(ids_graph, ids_eager)
     ids_dense, _ = llm.greedy_decode(dense, prompt, 20, use_graph=False)
     assert (ids_dense == ids_eager).float().mean() >= 0.8  # near-ties may flip an argmax
+
+
+# ---- the lean decode step: glue kernels against plain torch fp32, engine against the module path ----
+
+@pytest.mark.gpu
+def test_glue_kernels_match_torch_fp32():
+    ops = torch.ops.macko_spmv
+    torch.manual_seed(3)
+    for n in (64, 4096, 5000):
+        x = torch.randn(n, device="cuda", dtype=torch.float16)
+        w = (1 + 0.1 * torch.randn(n, device="cuda")).half()
+        want = x.float() * torch.rsqrt(x.float().pow(2).mean() + 1e-5) * w.float()
+        assert torch.allclose(ops.decode_rmsnorm(x, w, 1e-5).float(), want, rtol=2e-3, atol=2e-3)
+        g, u = torch.randn(n, device="cuda").half(), torch.randn(n, device="cuda").half()
+        want = torch.nn.functional.silu(g.float()) * u.float()
+        assert torch.allclose(ops.decode_silu_mul(g, u).float(), want, rtol=2e-3, atol=2e-3)
+    for n_heads, head_dim, max_len, pos in ((4, 64, 48, 0), (32, 128, 400, 37), (2, 16, 300, 299), (3, 96, 700, 511)):
+        H = n_heads * head_dim
+        q, k, v = (torch.randn(H, device="cuda").half() for _ in range(3))
+        inv = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda").float() / head_dim))
+        ang = torch.outer(torch.arange(max_len, device="cuda").float(), inv)
+        cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+        kc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+        vc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+        kc0, vc0 = kc.clone(), vc.clone()
+        position = torch.tensor([pos], device="cuda")
+        q_rot = ops.decode_rope_append(q, k, v, cos, sin, position, kc, vc)
+
+        def rope(t):  # rotate-half convention, fp32
+            t = t.float().view(n_heads, head_dim)
+            c, s = torch.cat((cos[pos], cos[pos])), torch.cat((sin[pos], sin[pos]))
+            rot = torch.cat((-t[:, head_dim // 2:], t[:, :head_dim // 2]), dim=1)
+            return t * c + rot * s
+
+        assert torch.allclose(q_rot.float().view(n_heads, head_dim), rope(q), rtol=2e-3, atol=2e-3)
+        assert torch.allclose(kc[:, pos].float(), rope(k), rtol=2e-3, atol=2e-3)
+        assert torch.equal(vc[:, pos], v.view(n_heads, head_dim))
+        keep = torch.ones(max_len, dtype=torch.bool, device="cuda")
+        keep[pos] = False
+        assert torch.equal(kc[:, keep], kc0[:, keep]) and torch.equal(vc[:, keep], vc0[:, keep])
+        scale = head_dim ** -0.5
+        out = ops.decode_attention(q_rot, kc, vc, position, scale).float().view(n_heads, head_dim)
+        att = torch.softmax(torch.einsum("hd,hpd->hp", q_rot.float().view(n_heads, head_dim),
+                                         kc[:, :pos + 1].float()) * scale, dim=-1)
+        want = torch.einsum("hp,hpd->hd", att, vc[:, :pos + 1].float())
+        assert torch.allclose(out, want, rtol=5e-3, atol=5e-3)
+
+
+@pytest.mark.gpu
+def test_concat_compressed_equals_compressing_the_stack():
+    torch.manual_seed(5)
+    mats = []
+    for rows in (7, 33, 64):
+        w = torch.randn(rows, 300, device="cuda", dtype=torch.float16)
+        w[torch.rand_like(w.float()) > 0.2] = 0
+        mats.append(w.contiguous())
+    mats[1][4] = 0  # an empty row inside
+    got = llm.concat_compressed([llm.macko_spmv.compress(m) for m in mats])
+    want = llm.macko_spmv.compress(torch.cat(mats, dim=0).contiguous())
+    assert got[3] == want[3] and got[4] == want[4]
+    for a, b in zip(got[:3], want[:3]):
+        assert a.dtype == b.dtype and torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sparse", [False, True])
+def test_engine_step_matches_module_forward(sparse):
+    torch.set_grad_enabled(False)
+    cfg = dict(n_layers=2, dim=256, hidden=688, n_heads=4, vocab=1000, max_len=64)
+    reference, _ = llm.build_model(0.5, sparse=False, **cfg)   # same seed -> same weights
+    consumed, _ = llm.build_model(0.5, sparse=sparse, **cfg)
+    engine = llm.DecodeEngine(consumed)
+    prompt = torch.randint(0, 1000, (1, 10), device="cuda")
+    want = reference(prompt, torch.arange(10, device="cuda"))[0].float()   # (10, vocab)
+    position = torch.zeros(1, dtype=torch.long, device="cuda")
+    for i in range(10):
+        logits = engine.step(prompt[0, i:i + 1].clone(), position).float()
+        assert torch.allclose(logits, want[i], rtol=3e-2, atol=3e-2), i
+        position.add_(1)
+    ids_graph, _ = llm.engine_decode(engine, prompt, 16, use_graph=True)
+    ids_eager, _ = llm.engine_decode(engine, prompt, 16, use_graph=False)
+    assert torch.equal(ids_graph, ids_eager)
+    ids_module, _ = llm.greedy_decode(reference, prompt, 16, use_graph=False)
+    assert (ids_module == ids_eager).float().mean() >= 0.8  # near-ties may flip an argmax
