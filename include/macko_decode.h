@@ -36,7 +36,7 @@ int macko_decode_rope_append_f16(const void *q, const void *k, const void *v,
 /*
  * Single-query attention per head over cache positions 0..*position:
  * out = softmax(scale * q K^T) V.  head_dim <= 256 and a multiple of 8, max_len <= 4096,
- * k_cache 16-byte aligned.
+ * both caches 16-byte aligned.
  */
 int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache,
                                const int64_t *position, void *out, int32_t n_heads,

@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
 {
     __shared__ float scores[kMaxLen];
     __shared__ float qs[256];
-    __shared__ float partial[kAttnThreads];
+    __shared__ float partial[kAttnThreads * 8];  // groups x head_dim <= 2048
     __shared__ float scratch[17];
     const int head = blockIdx.x, tid = threadIdx.x;
     long long pos = position[0];
@@ -126,13 +126,25 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
         local_sum += e;
     }
     const float inv = 1.0f / block_sum(local_sum, scratch);  // also orders the scores[] writes
-    // thread (g, d): dims d = tid % head_dim, position slices g = tid / head_dim
-    const int groups = kAttnThreads / head_dim > 0 ? kAttnThreads / head_dim : 1;
-    const int d = tid % head_dim, g = tid / head_dim;
-    float acc = 0.f;
-    if (g < groups)
-        for (int p = g; p < len; p += groups) acc += scores[p] * h2f(vh[(size_t)p * head_dim + d]);
-    partial[tid] = acc;
+    // Weighted sum of v: a thread owns 8 consecutive dims (one 16-byte load per position) of the
+    // positions p = g, g + groups, ...; the groups' partial sums meet in LDS.
+    const int lanes_per_row = head_dim >> 3;
+    const int groups = kAttnThreads / lanes_per_row;
+    const int g = tid / lanes_per_row, j = tid - g * lanes_per_row;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (g < groups) {
+        for (int p = g; p < len; p += groups) {
+            const float wgt = scores[p];
+            const u32x4 vv = reinterpret_cast<const u32x4 *>(vh + (size_t)p * head_dim)[j];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] += wgt * h2f((uint16_t)(vv[e] & 0xffffu));
+                acc[2 * e + 1] += wgt * h2f((uint16_t)(vv[e] >> 16));
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) partial[g * head_dim + 8 * j + e] = acc[e];
+    }
     __syncthreads();
     if (tid < head_dim) {
         float total = 0.f;
@@ -189,7 +201,8 @@ extern "C" int macko_decode_attention_f16(const void *q, const void *k_cache, co
     if (!q || !k_cache || !v_cache || !position || !out) return MACKO_E_INVALID_ARGUMENT;
     if (n_heads <= 0 || head_dim <= 0 || head_dim > 256 || (head_dim & 7) || max_len <= 0 || max_len > kMaxLen)
         return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(k_cache) & 15)) return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(k_cache) & 15) || (reinterpret_cast<uintptr_t>(v_cache) & 15))
+        return MACKO_E_INVALID_ARGUMENT;
     hipLaunchKernelGGL(attention_kernel, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
                        (const uint16_t *)q, (const uint16_t *)k_cache, (const uint16_t *)v_cache,
                        (const long long *)position, (uint16_t *)out, head_dim, max_len, scale);
