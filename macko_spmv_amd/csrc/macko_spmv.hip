@@ -94,27 +94,66 @@ __device__ __forceinline__ int load_row_window(const int *__restrict__ row_ptr, 
 
 // Smallest r in [0, rows] with row_ptr[r] >= target (rows if there is none), for two targets at
 // once.  All 64 lanes probe together.  window[k] is an already loaded probe (see
-// load_row_window) at base[k]; it resolves the search when rows carry similar entry counts,
-// otherwise 64-ary rounds follow.  Every value here is wave-uniform.
+// load_row_window) at base[k]; it resolves the search when rows carry similar entry counts.
+// Otherwise one more window is probed where the target should be if rows elsewhere are as long as
+// the ones just seen (which usually lands within a few rows even for very uneven matrices; that
+// window then replaces window[k] / base[k] so the caller finds its row starts in it), and 64-ary
+// rounds over what is still undecided follow.  Every value here is wave-uniform.
 __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_ptr, int rows, int lane,
-                                                  const int target[2], const int window[2], const int base[2],
+                                                  const int target[2], int (&window)[2], int (&base)[2],
                                                   int out[2])
 {
     int lo[2], hi[2];
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        const bool beyond = base[k] + lane > rows;
-        const unsigned long long m = __ballot(beyond || window[k] >= target[k]);
-        if (__builtin_expect(m == 0, 0)) {  // everything probed is below the target
-            lo[k] = base[k] + 64 > rows ? rows : base[k] + 64;
-            hi[k] = rows;
+    // narrows [lo, hi] with a window of row_ptr values: probed[i] >= target puts the answer at or
+    // before base + i, probed[i] < target puts it after
+    auto narrow = [&](int k, int probed, int at) {
+        const bool beyond = at + lane > rows;
+        const unsigned long long m = __ballot(beyond || probed >= target[k]);
+        if (m == 0) {
+            const int after = at + 64 > rows ? rows : at + 64;
+            lo[k] = lo[k] > after ? lo[k] : after;
         } else {
             const int f = __builtin_ctzll(m);
-            if (__builtin_expect(f == 0, 0)) {  // the answer is at or before the window start
-                lo[k] = 0;
-                hi[k] = base[k];
-            } else {
-                lo[k] = hi[k] = base[k] + f > rows ? rows : base[k] + f;
+            const int le = at + f > rows ? rows : at + f;
+            hi[k] = hi[k] < le ? hi[k] : le;
+            if (f > 0) lo[k] = lo[k] > le ? lo[k] : le;
+        }
+        if (lo[k] > hi[k]) lo[k] = hi[k];
+    };
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        lo[k] = 0;
+        hi[k] = rows;
+        narrow(k, window[k], base[k]);
+    }
+    if (__builtin_expect(lo[0] < hi[0] || lo[1] < hi[1], 0)) {
+        // second window, from the local row length: rows per entry around the first window
+        int probe[2], at[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            at[k] = base[k];
+            if (lo[k] < hi[k]) {
+                const int last = base[k] + 63 <= rows ? 63 : rows - base[k];
+                const int v0 = __builtin_amdgcn_readlane(window[k], 0);
+                const int v1 = __builtin_amdgcn_readlane(window[k], last);
+                const float per_entry = (float)(last > 0 ? last : 1) / (float)(v1 > v0 ? v1 - v0 : 1);
+                float jump = (float)(target[k] - v0) * per_entry;
+                jump = jump > 2.0e9f ? 2.0e9f : (jump < -2.0e9f ? -2.0e9f : jump);
+                long long g = (long long)base[k] + (long long)jump - 32;
+                const int gmax = rows - 63 > 0 ? rows - 63 : 0;
+                g = g < lo[k] - 1 ? lo[k] - 1 : g;  // stay inside what is still undecided
+                g = g > hi[k] - 32 ? hi[k] - 32 : g;
+                g = g < 0 ? 0 : (g > gmax ? gmax : g);
+                at[k] = (int)g;
+            }
+            probe[k] = load_row_window(row_ptr, rows, at[k], lane);  // both loads in flight together
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            if (lo[k] < hi[k]) {
+                narrow(k, probe[k], at[k]);
+                window[k] = probe[k];
+                base[k] = at[k];
             }
         }
     }
@@ -513,6 +552,8 @@ spmv_stream_kernel(const SpmvArgs a)
         r = uniform(range[0]);
         row_last = uniform(range[1]);
         have_work = r < row_last;
+        win_base = base[0];  // the search may have moved the windows
+        win = window[0];
         if (have_work) {  // first non-empty owned row; empty ones are written on the way
             slide_window(r);
             e0 = row_start(r);
@@ -529,8 +570,13 @@ spmv_stream_kernel(const SpmvArgs a)
                 e1 = row_start(r + 1);
             }
         }
-        if (have_work)  // end of my last owned row
-            s_end = row_last <= win_base + 63 ? row_start(row_last) : uniform(a.row_ptr[row_last]);
+        if (have_work) {  // end of my last owned row
+            if (row_last >= base[1] && row_last <= base[1] + 63)
+                s_end = __builtin_amdgcn_readlane(window[1], row_last - base[1]);
+            else
+                s_end = row_last >= win_base && row_last <= win_base + 63 ? row_start(row_last)
+                                                                            : uniform(a.row_ptr[row_last]);
+        }
     }
 
     // ---- 4. my tile range; the ring is filled with my first D tiles before x is even in LDS: they
