@@ -306,15 +306,24 @@ def main():
 
         hip = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
         hip.macko_calibration_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
-        read_pool = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+        def read_stride(nbytes):
+            return (int(nbytes) // 16 * 16 + 4095) // 4096 * 4096
+
+        # the pool holds at least two copies of the largest case, so consecutive launches never re-read
+        pool_bytes = max(1 << 30, 2 * max(read_stride(c["bytes"]) for c in cases))
+        read_pool = torch.ones(pool_bytes, dtype=torch.uint8, device="cuda")
         read_sink = torch.zeros(1, dtype=torch.int32, device="cuda")
 
+        def read_copies(nbytes):
+            return pool_bytes // read_stride(nbytes)
+
         def read_launches(nbytes):
-            # pure streaming read of the same number of bytes, rotating through 1 GiB
+            # pure streaming read of the same number of bytes, rotating through the pool
             nbytes = int(nbytes) // 16 * 16
-            stride = (nbytes + 4095) // 4096 * 4096
+            stride = read_stride(nbytes)
             sp = torch.cuda.current_stream().cuda_stream
-            for k in range(max(2, (1 << 30) // stride)):
+            for k in range(read_copies(nbytes)):
+                assert k * stride + nbytes <= pool_bytes  # the kernel trusts its arguments
                 rc = hip.macko_calibration_read(read_pool.data_ptr() + k * stride, nbytes, read_sink.data_ptr(), sp)
                 assert rc == 0, rc
 
@@ -332,7 +341,7 @@ def main():
             t_dense /= len(dense_copies)
             del dense_copies
             t_read, _ = time_graph(torch, lambda: read_launches(c["bytes"]), args.case_replays)
-            t_read /= max(2, (1 << 30) // ((int(c["bytes"]) // 16 * 16 + 4095) // 4096 * 4096))
+            t_read /= read_copies(c["bytes"])
             per_case.append({
                 "shape": f"{c['rows']}x{c['cols']}", "density": c["density"],
                 "macko_us": round(t_sparse * 1e6, 2), "dense_us": round(t_dense * 1e6, 2),

@@ -317,10 +317,11 @@ __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset,
                                            const u32x4 &buf_deltas)
 {
     static_assert(D == 1 || D == 2 || D == 4 || D == 8 || D == 16, "ring depth");
-    static_assert(VB == 2 || (VB == 1 && D == 2), "the int8 ring exists at depth 2 only");
+    static_assert(VB == 2 || (VB == 1 && D <= 2), "the int8 ring exists at depth 1 and 2 only");
     if (VB == 1) {
-        if (J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v96", MACKO_FIXED_CLOBBERS_4);
-        if (J == 1) MACKO_RING_ISSUE_I8("v[92:93]", "v97", MACKO_FIXED_CLOBBERS_4);
+        if (D == 1 && J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v92", MACKO_FIXED_CLOBBERS_4);
+        if (D == 2 && J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v96", MACKO_FIXED_CLOBBERS_4);
+        if (D == 2 && J == 1) MACKO_RING_ISSUE_I8("v[92:93]", "v97", MACKO_FIXED_CLOBBERS_4);
         return;
     }
     if (D == 1 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v92", MACKO_FIXED_CLOBBERS_4);
@@ -801,7 +802,6 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 
     const Tuning t = g_tuning;
     const int block = t.block ? t.block : 1024;
-    const int depth = t.depth ? t.depth : 2;
     const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
     const int waves = block / kWave;
     // about one wave per tile at most, so tiny matrices get a small grid; but when rows are about
@@ -813,20 +813,27 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     long long grid = (waves_wanted + waves - 1) / waves;
     if (grid > (long long)info.compute_units * wg_per_cu) grid = (long long)info.compute_units * wg_per_cu;
     if (grid < 1) grid = 1;
+    // Ring depth: one tile in flight behind the one being processed is enough, and cheapest to
+    // start, when a wave owns a single row or only a few tiles; waves that walk many tiles over
+    // several rows do slightly better with two (measured on the Llama shapes; deeper is slower).
+    const long long n_waves = grid * waves;
+    const int depth = t.depth ? t.depth : ((long long)a.rows > n_waves && n_tiles >= 6 * n_waves ? 2 : 1);
 
     const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
     if (lds_need > (size_t)info.max_lds_bytes)
         return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
-    if (VB == 1) {  // int8 values: the default launch shape only
+    if (VB == 1) {  // int8 values: the default launch shapes only
         if (block == 1024 && depth == 2)
             return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_need, stream);
+        if (block == 1024 && depth == 1)
+            return launch_stream<1024, 1, true, AXPBY, VB>(a, (int)grid, lds_need, stream);
         return MACKO_E_INVALID_ARGUMENT;
     }
 #define MACKO_CASE(B, D_) \
     if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
     MACKO_CASE(1024, 2)
+    MACKO_CASE(1024, 1)
     if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
-        MACKO_CASE(1024, 1)
         MACKO_CASE(1024, 4)
         MACKO_CASE(1024, 8)
         MACKO_CASE(512, 2)
