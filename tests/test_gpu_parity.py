@@ -219,6 +219,32 @@ def test_multiply_rows_of_wildly_different_length():
     _check_product(dense, x, label="wild")
 
 
+def test_multiply_rows_not_more_than_waves():
+    # ownership by proportional row share: one row per wave, with empty rows in between, few rows
+    # over many tiles (most waves idle), and exactly as many rows as the launch has waves
+    rng = np.random.default_rng(21)
+    for rows, cols, density in [(4096, 600, 0.3), (4096, 3000, 0.05), (300, 40000, 0.3), (4095, 2049, 0.5),
+                                (17, 30000, 0.9), (2048, 8192, 0.2)]:
+        dense = helpers.random_sparse(rng, rows, cols, density, scale=0.05)
+        dense[rng.random(rows) < 0.1] = 0  # empty rows, also first / last now and then
+        dense[0] = 0
+        x = rng.standard_normal(cols).astype(np.float16)
+        _check_product(dense, x, label=f"row share {rows}x{cols}")
+
+
+def test_multiply_row_lengths_sorted():
+    # row lengths grow monotonically, so the proportional row guess is far off for every wave and
+    # the search runs through its second window and the 64-ary rounds
+    rng = np.random.default_rng(22)
+    for rows, cols in [(9000, 2048), (20000, 512), (5000, 4096)]:
+        density = np.linspace(0.002, 0.9, rows) ** 2
+        dense = (rng.standard_normal((rows, cols), dtype=np.float32) * 0.05).astype(np.float16)
+        dense[rng.random((rows, cols)) >= density[:, None]] = 0
+        x = rng.standard_normal(cols).astype(np.float16)
+        _check_product(dense, x, label=f"sorted rows {rows}x{cols}")
+        _check_product(dense[::-1].copy(), x, label=f"sorted rows reversed {rows}x{cols}")
+
+
 def test_multiply_x_longer_than_cols_and_unaligned():
     rng = np.random.default_rng(9)
     dense = helpers.random_sparse(rng, 128, 1001, 0.4, scale=1.0)
