@@ -256,8 +256,6 @@ __device__ __forceinline__ u32x4 make_buffer(const void *base, u32 bytes)
     return r;
 }
 
-#define MACKO_FIXED_CLOBBERS_16 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167"
-#define MACKO_FIXED_CLOBBERS_8 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127"
 #define MACKO_FIXED_CLOBBERS_4 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107"
 
 // row_ptr probe k (k = 0, 1) -> v78 + k
@@ -316,7 +314,7 @@ template <int D, int J, int VB>
 __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
                                            const u32x4 &buf_deltas)
 {
-    static_assert(D == 1 || D == 2 || D == 4 || D == 8 || D == 16, "ring depth");
+    static_assert(D == 1 || D == 2 || D == 4, "ring depth");
     static_assert(VB == 2 || (VB == 1 && D <= 2), "the int8 ring exists at depth 1 and 2 only");
     if (VB == 1) {
         if (D == 1 && J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v92", MACKO_FIXED_CLOBBERS_4);
@@ -331,30 +329,6 @@ __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset,
     if (D == 4 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v105", MACKO_FIXED_CLOBBERS_4);
     if (D == 4 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v106", MACKO_FIXED_CLOBBERS_4);
     if (D == 4 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v107", MACKO_FIXED_CLOBBERS_4);
-    if (D == 8 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v120", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v121", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v122", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v123", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 4) MACKO_RING_ISSUE("v[104:107]", "v124", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 5) MACKO_RING_ISSUE("v[108:111]", "v125", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 6) MACKO_RING_ISSUE("v[112:115]", "v126", MACKO_FIXED_CLOBBERS_8);
-    if (D == 8 && J == 7) MACKO_RING_ISSUE("v[116:119]", "v127", MACKO_FIXED_CLOBBERS_8);
-    if (D == 16 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v152", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v153", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v154", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v155", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 4) MACKO_RING_ISSUE("v[104:107]", "v156", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 5) MACKO_RING_ISSUE("v[108:111]", "v157", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 6) MACKO_RING_ISSUE("v[112:115]", "v158", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 7) MACKO_RING_ISSUE("v[116:119]", "v159", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 8) MACKO_RING_ISSUE("v[120:123]", "v160", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 9) MACKO_RING_ISSUE("v[124:127]", "v161", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 10) MACKO_RING_ISSUE("v[128:131]", "v162", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 11) MACKO_RING_ISSUE("v[132:135]", "v163", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 12) MACKO_RING_ISSUE("v[136:139]", "v164", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 13) MACKO_RING_ISSUE("v[140:143]", "v165", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 14) MACKO_RING_ISSUE("v[144:147]", "v166", MACKO_FIXED_CLOBBERS_16);
-    if (D == 16 && J == 15) MACKO_RING_ISSUE("v[148:151]", "v167", MACKO_FIXED_CLOBBERS_16);
 }
 
 template <int D, int J, int N>
@@ -367,30 +341,6 @@ __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
     if (D == 4 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v105");
     if (D == 4 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v106");
     if (D == 4 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v107");
-    if (D == 8 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v120");
-    if (D == 8 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v121");
-    if (D == 8 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v122");
-    if (D == 8 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v123");
-    if (D == 8 && J == 4) MACKO_RING_TAKE("v104", "v105", "v106", "v107", "v124");
-    if (D == 8 && J == 5) MACKO_RING_TAKE("v108", "v109", "v110", "v111", "v125");
-    if (D == 8 && J == 6) MACKO_RING_TAKE("v112", "v113", "v114", "v115", "v126");
-    if (D == 8 && J == 7) MACKO_RING_TAKE("v116", "v117", "v118", "v119", "v127");
-    if (D == 16 && J == 0) MACKO_RING_TAKE("v88", "v89", "v90", "v91", "v152");
-    if (D == 16 && J == 1) MACKO_RING_TAKE("v92", "v93", "v94", "v95", "v153");
-    if (D == 16 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v154");
-    if (D == 16 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v155");
-    if (D == 16 && J == 4) MACKO_RING_TAKE("v104", "v105", "v106", "v107", "v156");
-    if (D == 16 && J == 5) MACKO_RING_TAKE("v108", "v109", "v110", "v111", "v157");
-    if (D == 16 && J == 6) MACKO_RING_TAKE("v112", "v113", "v114", "v115", "v158");
-    if (D == 16 && J == 7) MACKO_RING_TAKE("v116", "v117", "v118", "v119", "v159");
-    if (D == 16 && J == 8) MACKO_RING_TAKE("v120", "v121", "v122", "v123", "v160");
-    if (D == 16 && J == 9) MACKO_RING_TAKE("v124", "v125", "v126", "v127", "v161");
-    if (D == 16 && J == 10) MACKO_RING_TAKE("v128", "v129", "v130", "v131", "v162");
-    if (D == 16 && J == 11) MACKO_RING_TAKE("v132", "v133", "v134", "v135", "v163");
-    if (D == 16 && J == 12) MACKO_RING_TAKE("v136", "v137", "v138", "v139", "v164");
-    if (D == 16 && J == 13) MACKO_RING_TAKE("v140", "v141", "v142", "v143", "v165");
-    if (D == 16 && J == 14) MACKO_RING_TAKE("v144", "v145", "v146", "v147", "v166");
-    if (D == 16 && J == 15) MACKO_RING_TAKE("v148", "v149", "v150", "v151", "v167");
 }
 template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
@@ -782,7 +732,7 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 // Launch-shape overrides for tuning runs (0 = built-in default).  Not part of the public ABI.
 struct Tuning {
     int block;      // threads per workgroup: 256, 512 or 1024
-    int depth;      // tiles in flight per wave: 1, 2, 4 or 8 (not every block size has every depth)
+    int depth;      // tiles in flight per wave: 1, 2 or 4 (4 only with 1024 threads, 1 only with 1024)
     int wg_per_cu;  // workgroups launched per compute unit
 };
 Tuning g_tuning = {0, 0, 0};
@@ -835,11 +785,8 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     MACKO_CASE(1024, 1)
     if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
         MACKO_CASE(1024, 4)
-        MACKO_CASE(1024, 8)
         MACKO_CASE(512, 2)
-        MACKO_CASE(512, 4)
         MACKO_CASE(256, 2)
-        MACKO_CASE(256, 4)
     }
 #undef MACKO_CASE
     return MACKO_E_INVALID_ARGUMENT;
