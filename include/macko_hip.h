@@ -81,6 +81,18 @@ int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
                             int64_t padded_entries, void *stream);
 
 /*
+ * Y[b, :] = M X[b, :] for b < batch.  X is [batch, ldx] and Y [batch, ldy], row-major fp16 with
+ * ldx >= cols and ldy >= rows (elements).  The matrix is streamed once per group of up to four
+ * vectors (as many as fit next to each other in LDS), the rest like macko_spmv_f16.  No
+ * counterpart in the upstream package, whose LLM runner maps the single-vector operator over
+ * the batch dimension (python_scripts/util_run_pruned_llm.py:112-118).
+ */
+int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t *row_ptr,
+                           const void *x, void *y, int32_t rows, int32_t cols,
+                           int64_t padded_entries, int32_t batch, int64_t ldx, int64_t ldy,
+                           void *stream);
+
+/*
  * int8 values variant.  Same arrays, except that `values` holds int8 [P] (8-byte aligned) and
  * `dense` is a row-major int8 matrix.  The compressor pair replaces compress_rows_int8_cpu
  * (src/macko_spmv/cuda/cpu_compressor.cuh:75-117), which differs from the fp16 one in keeping

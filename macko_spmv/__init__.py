@@ -9,6 +9,7 @@ from macko_spmv_amd import (  # noqa: F401
     move_to_device,
     multiply,
     multiply_axpby,
+    multiply_batched,
     multiply_int8,
     multiply_int8_axpby,
 )

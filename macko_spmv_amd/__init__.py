@@ -50,6 +50,11 @@ def _multiply_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
     return torch.empty((M_rows,), device=M_values.device, dtype=M_values.dtype)
 
 
+@torch.library.register_fake("macko_spmv::multiply_batched")
+def _multiply_batched_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, X):
+    return torch.empty((X.shape[0], M_rows), device=M_values.device, dtype=M_values.dtype)
+
+
 @torch.library.register_fake("macko_spmv::multiply_axpby")
 def _multiply_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C, alpha, beta):
     return None
@@ -111,6 +116,15 @@ def multiply(compressed_M, V):
         compressed_M[4],
         V,
     )
+
+
+def multiply_batched(compressed_M, X):
+    """Y[b] = M @ X[b] for X of shape (batch, cols) -> (batch, rows).  The matrix is read once per
+    group of up to four vectors.  Upstream has only the single-vector operator and maps it over
+    the batch dimension (python_scripts/util_run_pruned_llm.py:112-118)."""
+    assert compressed_M[0].is_cuda and X.is_cuda
+    assert X.dim() == 2 and X.is_contiguous()
+    return torch.ops.macko_spmv.multiply_batched.default(*compressed_M[:5], X)
 
 
 def multiply_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):

@@ -50,6 +50,8 @@ struct SpmvArgs {
     // [floor(w*rows/W), floor((w+1)*rows/W)), at most one row each.  No split of whole rows can do
     // better than the longest row, and cutting by entries could hand one wave two rows.
     u32 row_even;
+    // batched product (NB > 1 vectors per launch): elements between consecutive vectors of x / y
+    int ldx, ldy;
 #ifdef MACKO_SPMV_TRACE
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif
@@ -342,12 +344,18 @@ __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
     if (D == 4 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v106");
     if (D == 4 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v107");
 }
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB>
+// NB = vectors multiplied per launch (1, 2 or 4).  With NB > 1 the NB copies of x are interleaved in
+// LDS (element c of vector b at half-word c * NB + b), so one LDS read per stored entry fetches the
+// operand of every vector, and a row ends with NB sums.  NB > 1 exists for fp16 values, x in LDS,
+// plain product only.
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
+    static_assert(NB == 1 || (NB <= 4 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int WAVES = BLOCK / kWave;
+    constexpr int kBatchShift = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
     constexpr int kTileLoads = 2 * D;  // tracked loads per full ring
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -390,7 +398,7 @@ spmv_stream_kernel(const SpmvArgs a)
         probe_issue<1>((u32)i1 * 4, buf_rows);
     }
     const u32x4 buf_x = make_buffer(a.x, (u32)x_nvec * 16);  // past the end reads as zero
-    if (X_LDS) {
+    if (X_LDS && NB == 1) {
         xpiece_issue<0>((u32)tid * 16, buf_x);
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
@@ -402,7 +410,25 @@ spmv_stream_kernel(const SpmvArgs a)
     // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
     //         x, goes to LDS through ordinary loads (rare: more than 16384 columns, or an x that is
     //         not 16-byte aligned) ------------------------------------------------------------------
-    if (X_LDS) {
+    if (NB > 1) {
+        // every vector through ordinary loads, interleaved: element c of vector b at dst[c * NB + b]
+        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront * NB);
+        const bool vec_ok = x_vec && (a.ldx & 7) == 0;
+        const int nvec = vec_ok ? a.cols >> 3 : 0;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint16_t *xb = a.x + (size_t)b * (size_t)a.ldx;
+            for (int i = tid; i < nvec; i += BLOCK) {
+                const u32x4 v = reinterpret_cast<const u32x4 *>(xb)[i];
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    dst[(8 * i + e) * NB + b] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+            }
+            for (int i = (nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i * NB + b] = xb[i];
+        }
+        if (tid < kLdsFront * NB / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
+        if (tid < kLdsBack * NB / 2) dst[a.cols * NB + tid] = 0;
+    } else if (X_LDS) {
         uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
         u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
         if (__builtin_expect(x_nvec > kXRegs * BLOCK, 0))
@@ -415,7 +441,7 @@ spmv_stream_kernel(const SpmvArgs a)
     MACKO_STAMP(1);
 
     // ---- 3. which rows are mine -----------------------------------------------------------------------
-    constexpr int kXLoads = X_LDS ? kXRegs : 0;
+    constexpr int kXLoads = X_LDS && NB == 1 ? kXRegs : 0;
     int window[2];
     window[0] = probe_take<0, kXLoads + 1>();
     window[1] = probe_take<1, kXLoads>();
@@ -431,12 +457,17 @@ spmv_stream_kernel(const SpmvArgs a)
             win = load_row_window(a.row_ptr, a.rows, win_base, lane);
         }
     };
-    auto store_row = [&](int r, float total) {
+    auto store_row = [&](int r, float total, int b = 0) {
         if (lane == 0) {
             float out = total;
-            if (AXPBY) out = a.alpha * total + a.beta * half_bits_to_float(a.y[r]);
-            a.y[r] = float_to_half_bits(out);
+            uint16_t *y = NB == 1 ? a.y : a.y + (size_t)b * (size_t)a.ldy;
+            if (AXPBY) out = a.alpha * total + a.beta * half_bits_to_float(y[r]);
+            y[r] = float_to_half_bits(out);
         }
+    };
+    auto store_empty_row = [&](int r) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) store_row(r, 0.f, b);
     };
 
     int row_last = 0;
@@ -510,7 +541,7 @@ spmv_stream_kernel(const SpmvArgs a)
             e0 = row_start(r);
             e1 = row_start(r + 1);
             while (e1 == e0) {
-                store_row(r, 0.f);
+                store_empty_row(r);
                 ++r;
                 if (r >= row_last) {
                     have_work = false;
@@ -543,7 +574,9 @@ spmv_stream_kernel(const SpmvArgs a)
     }
 
     // ---- 5. x pieces into LDS (older than the ring loads just issued, if any) ---------------------------
-    if (X_LDS) {
+    if (NB > 1) {
+        __syncthreads();
+    } else if (X_LDS) {
         const u32 lds_x = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
         const u32 dst0 = lds_x + (u32)tid * 16, dst1 = dst0 + BLOCK * 16;
         if (__builtin_expect(have_work, 1)) {
@@ -564,12 +597,17 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 6. stream ----------------------------------------------------------------------------------
     float acc0 = 0.f, acc1 = 0.f;
+    float accb[NB > 1 ? NB : 1] = {};  // batched variant: one accumulator per vector
     typedef __attribute__((address_space(3))) const uint16_t *lds_u16_ptr;
-    // LDS byte address of x[0] (x sits kLdsFront bytes into this kernel's dynamic LDS)
-    const u32 x_addr = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
+    typedef __attribute__((address_space(3))) const u32 *lds_u32_ptr;
+    typedef __attribute__((address_space(3))) const u32x2 *lds_u32x2_ptr;
+    // LDS byte address of x[0] (x sits kLdsFront bytes, times NB, into this kernel's dynamic LDS)
+    const u32 x_addr = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront * NB;
     // row_addr: LDS byte address the next entry of the current row would read if its nibble were 0,
-    // i.e. x_addr + 2 * (entries of the row consumed so far + their nibble sum).  Wave-uniform.
-    u32 row_addr = x_addr;
+    // i.e. row_origin + 2 * (entries of the row consumed so far + their nibble sum).  Wave-uniform.
+    // With NB > 1 it stays relative to x (row_origin = 0) and is scaled by NB when an entry is read.
+    const u32 row_origin = NB == 1 ? x_addr : 0u;
+    u32 row_addr = row_origin;
     MACKO_STAMP(5);
 
     // The eight multiply-adds of a lane: entry k reads x at base + 2k + 2 * (nibbles 0..k), which is
@@ -579,6 +617,23 @@ spmv_stream_kernel(const SpmvArgs a)
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const u32 addr = __builtin_amdgcn_udot8(dd, m[k], base, false);
+            if (NB > 1) {
+                const u32 w = vv[k >> 1];
+                const float mv = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+                const u32 at = x_addr + (addr << kBatchShift) + ((2 * k) << kBatchShift);
+                if (NB == 2) {
+                    const u32 xs = *reinterpret_cast<lds_u32_ptr>(at);
+                    accb[0] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs & 0xffffu)), accb[0]);
+                    accb[1] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs >> 16)), accb[1]);
+                } else {
+                    const u32x2 xs = *reinterpret_cast<lds_u32x2_ptr>(at);
+                    accb[0] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.x & 0xffffu)), accb[0]);
+                    accb[1] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.x >> 16)), accb[1]);
+                    accb[2 % NB] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.y & 0xffffu)), accb[2 % NB]);
+                    accb[3 % NB] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.y >> 16)), accb[3 % NB]);
+                }
+                continue;
+            }
             uint16_t xb;
 #if defined(MACKO_EXP_NO_GATHER)
             xb = (uint16_t)(addr & 0x3fffu);
@@ -648,16 +703,24 @@ spmv_stream_kernel(const SpmvArgs a)
     };
 
     auto finish_row = [&]() {
-        store_row(r, wave_sum(acc0 + acc1));
-        acc0 = acc1 = 0.f;
-        row_addr = x_addr;
+        if (NB == 1) {
+            store_row(r, wave_sum(acc0 + acc1));
+            acc0 = acc1 = 0.f;
+        } else {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                store_row(r, wave_sum(accb[b]), b);
+                accb[b] = 0.f;
+            }
+        }
+        row_addr = row_origin;
         do {  // next non-empty owned row; empty ones get their zero on the way
             ++r;
             if (r >= row_last) break;  // then the row just finished ended at s_end and all loops end
             slide_window(r);
             e0 = row_start(r);
             e1 = row_start(r + 1);
-            if (e1 == e0) store_row(r, 0.f);
+            if (e1 == e0) store_empty_row(r);
         } while (e1 == e0);
     };
 
@@ -702,10 +765,10 @@ __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2>
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1>
 int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB>;
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
     a.entries_q = (u32)(a.padded / n_waves);
     a.entries_rem = (u32)(a.padded % n_waves);
@@ -737,7 +800,7 @@ struct Tuning {
 };
 Tuning g_tuning = {0, 0, 0};
 
-template <bool AXPBY, int VB = 2>
+template <bool AXPBY, int VB = 2, int NB = 1>
 int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 {
     if (a.rows == 0) return 0;
@@ -769,7 +832,12 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     const long long n_waves = grid * waves;
     const int depth = t.depth ? t.depth : ((long long)a.rows > n_waves && n_tiles >= 6 * n_waves ? 2 : 1);
 
-    const size_t lds_need = (size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack;
+    const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack);
+    if (NB > 1) {  // NB vectors per launch: the caller has checked that they fit in LDS
+        if (lds_need > (size_t)info.max_lds_bytes || block != 1024) return MACKO_E_INVALID_ARGUMENT;
+        if (depth == 2) return launch_stream<1024, 2, true, false, 2, NB>(a, (int)grid, lds_need, stream);
+        return launch_stream<1024, 1, true, false, 2, NB>(a, (int)grid, lds_need, stream);
+    }
     if (lds_need > (size_t)info.max_lds_bytes)
         return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
     if (VB == 1) {  // int8 values: the default launch shapes only
@@ -831,7 +899,8 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0,             0,
+               0,                   0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = g_trace;
 #endif
@@ -847,7 +916,8 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0,             0,
+               0,                   0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
@@ -863,7 +933,8 @@ extern "C" int macko_spmv_i8f16(const void *values, const void *deltas, const in
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, 1.0f,          0.0f,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0,             0,
+               0,                   0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
@@ -879,9 +950,56 @@ extern "C" int macko_spmv_i8f16_axpby(const void *values, const void *deltas, co
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows,                cols,                padded_entries, alpha,         beta,
-               0,                   0,                   0,              0,             0};
+               0,                   0,                   0,              0,             0,
+               0,                   0};
 #ifdef MACKO_SPMV_TRACE
     a.trace = nullptr;
 #endif
     return spmv_dispatch<true, 1>(a, as_stream(stream));
+}
+
+// Y[b, :] = M X[b, :] for `batch` vectors: X is [batch, ldx] and Y [batch, ldy] row-major fp16
+// (ldx >= cols, ldy >= rows).  The matrix is streamed once per group of up to four vectors (as
+// many as fit in LDS next to each other), so the cost per vector drops accordingly.  The upstream
+// package has no batched entry: its LLM runner maps the single-vector operator over the batch
+// dimension (python_scripts/util_run_pruned_llm.py:112-118).
+extern "C" int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t *row_ptr,
+                                      const void *x, void *y, int32_t rows, int32_t cols,
+                                      int64_t padded_entries, int32_t batch, int64_t ldx, int64_t ldy,
+                                      void *stream)
+{
+    using namespace macko;
+    if (batch < 0 || ldx < cols || ldy < rows || ldx >= (1ll << 31) || ldy >= (1ll << 31))
+        return MACKO_E_INVALID_ARGUMENT;
+    if (batch == 0) return 0;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
+    if (rc != 0) return rc;
+    DeviceInfo info;
+    rc = device_info(&info);
+    if (rc != 0) return rc;
+    const size_t per_vector = (size_t)kLdsFront + 2 * (size_t)cols + kLdsBack;
+    int done = 0;
+    while (done < batch) {
+        const int left = batch - done;
+        SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr,
+                   (const uint16_t *)x + (size_t)done * (size_t)ldx, (uint16_t *)y + (size_t)done * (size_t)ldy,
+                   rows, cols, padded_entries, 1.0f, 0.0f, 0, 0, 0, 0, 0, (int)ldx, (int)ldy};
+#ifdef MACKO_SPMV_TRACE
+        a.trace = nullptr;
+#endif
+        int step;
+        if (padded_entries > 0 && left >= 4 && 4 * per_vector <= (size_t)info.max_lds_bytes) {
+            step = 4;
+            rc = spmv_dispatch<false, 2, 4>(a, as_stream(stream));
+        } else if (padded_entries > 0 && left >= 2 && 2 * per_vector <= (size_t)info.max_lds_bytes) {
+            step = 2;
+            rc = spmv_dispatch<false, 2, 2>(a, as_stream(stream));
+        } else {
+            step = 1;
+            rc = spmv_dispatch<false>(a, as_stream(stream));
+        }
+        if (rc != 0) return rc;
+        done += step;
+    }
+    return 0;
 }

@@ -53,6 +53,31 @@ at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
     return C;
 }
 
+// Y[b] = M @ X[b] for X of shape [batch, M_cols] -> [batch, M_rows].
+at::Tensor multiply_batched_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                                const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &X)
+{
+    TORCH_CHECK(M_values.dtype() == at::kHalf && X.dtype() == at::kHalf, "M and X must be torch.half");
+    TORCH_CHECK(M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt, "bad index dtypes");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && X.is_cuda(),
+                "all tensors must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
+                    X.is_contiguous(),
+                "all tensors must be contiguous");
+    TORCH_CHECK(X.dim() == 2 && X.size(1) >= M_cols, "X must be [batch, >= M_cols]");
+    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
+    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
+    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    at::Tensor Y = at::empty({X.size(0), M_rows}, M_values.options());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    check_rc(macko_spmv_f16_batched(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                    X.data_ptr(), Y.data_ptr(), (int32_t)M_rows, (int32_t)M_cols, M_values.numel(),
+                                    (int32_t)X.size(0), X.size(1), M_rows, (void *)stream),
+             "multiply_batched");
+    return Y;
+}
+
 // C = alpha * (M @ V) + beta * C, in place on C.
 void multiply_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
                         int64_t M_rows, int64_t M_cols, const at::Tensor &V, at::Tensor C, double alpha,
@@ -301,6 +326,8 @@ TORCH_LIBRARY(macko_spmv, m)
 {
     // same schema string as the upstream package
     m.def("multiply(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, Tensor V) -> Tensor");
+    m.def("multiply_batched(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor X) -> Tensor");
     m.def("multiply_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
           "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
     m.def("compress(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
@@ -320,6 +347,7 @@ TORCH_LIBRARY(macko_spmv, m)
 TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
 {
     m.impl("multiply", &multiply_hip);
+    m.impl("multiply_batched", &multiply_batched_hip);
     m.impl("multiply_axpby", &multiply_axpby_hip);
     m.impl("compress", &compress_hip);
     m.impl("compress_int8", &compress_int8_hip);

@@ -68,8 +68,8 @@ class MackoLinear(nn.Module):
         compressed = (self.c_0, self.c_1, self.c_2, self.c_3, self.c_4)
         if flat.shape[0] == 1:
             out = macko_spmv.multiply(compressed, flat[0].contiguous()).unsqueeze(0)
-        else:  # one product per row of x, as the upstream vmap fallback does
-            out = torch.stack([macko_spmv.multiply(compressed, row.contiguous()) for row in flat])
+        else:  # all rows of x in one call; upstream maps the single-vector operator over them (vmap)
+            out = macko_spmv.multiply_batched(compressed, flat.contiguous())
         return out.reshape(*lead, self.c_3)
 
     def weight_bytes(self):

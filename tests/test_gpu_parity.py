@@ -245,6 +245,58 @@ def test_multiply_row_lengths_sorted():
         _check_product(dense[::-1].copy(), x, label=f"sorted rows reversed {rows}x{cols}")
 
 
+@pytest.mark.parametrize("rows,cols,density", [(257, 1500, 0.3), (4096, 4096, 0.5), (11008, 4096, 0.1),
+                                               (64, 20000, 0.2), (300, 515, 0.9), (1000, 70000, 0.05),
+                                               (33, 90000, 0.1), (512, 512, 0.0)])
+def test_multiply_batched(rows, cols, density):
+    # every vector of the batch against the dense float64 product and against the single-vector path;
+    # batch sizes cover the 4-, 2- and 1-vector launches and their combinations, and LDS limits
+    # (70000 columns: two vectors per launch; 90000: one)
+    rng = np.random.default_rng(rows + cols)
+    dense = helpers.random_sparse(rng, rows, cols, density, scale=0.05)
+    if rows > 40:
+        dense[3] = 0
+        dense[-1] = 0
+    compressed = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    for batch in (1, 2, 3, 4, 5, 7, 8):
+        X = rng.standard_normal((batch, cols)).astype(np.float16)
+        Xg = torch.from_numpy(X).cuda()
+        print("batched case", rows, cols, density, batch, flush=True)
+        Y = macko_spmv.multiply_batched(compressed, Xg)
+        assert Y.shape == (batch, rows) and Y.dtype == torch.float16
+        Y_np = Y.cpu().numpy()
+        for b in range(batch):
+            helpers.assert_close_fp16(Y_np[b], helpers.dense_reference(dense, X[b]))
+            single = macko_spmv.multiply(compressed, Xg[b]).cpu().numpy()
+            assert np.allclose(Y_np[b].astype(np.float32), single.astype(np.float32), rtol=1e-2, atol=1e-3)
+
+
+def test_multiply_batched_strided_through_c_abi():
+    # leading dimensions larger than cols / rows, odd ldx (unaligned vectors take the scalar copy)
+    rng = np.random.default_rng(77)
+    rows, cols, batch, ldx, ldy = 500, 1001, 6, 1013, 512
+    dense = helpers.random_sparse(rng, rows, cols, 0.3, scale=0.05)
+    c = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    X = rng.standard_normal((batch, ldx)).astype(np.float16)
+    Xg = torch.from_numpy(X).cuda()
+    Yg = torch.full((batch, ldy), 7.0, dtype=torch.float16, device="cuda")
+    lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
+    vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+    lib.macko_spmv_f16_batched.argtypes = [vp, vp, vp, vp, vp, i32, i32, i64, i32, i64, i64, vp]
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.macko_spmv_f16_batched(c[0].data_ptr(), c[1].data_ptr(), c[2].data_ptr(), Xg.data_ptr(), Yg.data_ptr(),
+                                    rows, cols, c[0].numel(), batch, ldx, ldy, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    Y = Yg.cpu().numpy()
+    for b in range(batch):
+        helpers.assert_close_fp16(Y[b, :rows], helpers.dense_reference(dense, X[b, :cols]))
+    assert (Y[:, rows:] == 7.0).all()  # nothing written past the rows
+    # leading dimensions smaller than the matrix are rejected before any launch
+    assert lib.macko_spmv_f16_batched(c[0].data_ptr(), c[1].data_ptr(), c[2].data_ptr(), Xg.data_ptr(), Yg.data_ptr(),
+                                      rows, cols, c[0].numel(), batch, cols - 1, ldy, stream) == -1
+
+
 def test_multiply_x_longer_than_cols_and_unaligned():
     rng = np.random.default_rng(9)
     dense = helpers.random_sparse(rng, 128, 1001, 0.4, scale=1.0)
