@@ -200,6 +200,7 @@ def main():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
     ap.add_argument("--no-compress", action="store_true", help="skip the compressor timing")
     ap.add_argument("--no-int8", action="store_true", help="skip the int8-values variant timing")
+    ap.add_argument("--no-batched", action="store_true", help="skip the batched-product timing")
     ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
     ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
                     help="llama = the headline workload; large / skew = the other shape families")
@@ -379,6 +380,26 @@ def main():
             })
             log("int8:", int8_cases[-1])
 
+    # ---- batched product (several vectors per pass over the matrix), density 0.5 cases -------------
+    batched_cases = []
+    if not args.no_batched:
+        for c in cases:
+            if c["density"] != 0.5:
+                continue
+            n_copies = max(2, min(64, int(1.0e9 // c["bytes"]) + 1))
+            copies = c["copies"] + [clone_compressed(c["copies"][0]) for _ in range(n_copies - 2)]
+            entry = {"shape": f"{c['rows']}x{c['cols']}", "density": c["density"]}
+            for batch in (1, 2, 4, 8):
+                X = torch.randn(batch, c["cols"], device="cuda").half()
+                t, _ = time_graph(torch, lambda: [mk.multiply_batched(cc, X) for cc in copies], args.case_replays)
+                t /= len(copies)
+                td, _ = time_graph(torch, lambda: [torch.matmul(X, c["W"].t()) for _ in range(4)], args.case_replays)
+                entry[f"b{batch}_us"] = round(t * 1e6, 2)
+                entry[f"b{batch}_dense_us"] = round(td * 1e6 / 4, 2)
+            del copies
+            batched_cases.append(entry)
+            log("batched:", entry)
+
     # ---- the compressor: whole compress() call (count pass, read-back of the total, fill pass) -----
     compress_cases = []
     if not args.no_compress:
@@ -464,6 +485,7 @@ def main():
         "cases": per_case,
         "compress": compress_cases,
         "int8_values_variant": int8_cases,
+        "batched_product": batched_cases,
         "device": dev.name,
     }
     print(json.dumps(out), flush=True)

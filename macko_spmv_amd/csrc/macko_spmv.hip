@@ -415,15 +415,30 @@ spmv_stream_kernel(const SpmvArgs a)
         uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront * NB);
         const bool vec_ok = x_vec && (a.ldx & 7) == 0;
         const int nvec = vec_ok ? a.cols >> 3 : 0;
+        // 8 columns of every vector per thread and step: NB 16-byte loads, interleaved in registers,
+        // written back as NB 16-byte stores (16 * NB contiguous bytes of LDS)
+        for (int i = tid; i < nvec; i += BLOCK) {
+            u32x4 v[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                v[b] = reinterpret_cast<const u32x4 *>(a.x + (size_t)b * (size_t)a.ldx)[i];
+            u32 out[4 * NB];  // half-word (c * NB + b) = element c of vector b
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+#pragma unroll
+                for (int b = 0; b < NB; b += 2) {
+                    const u32 lo = (v[b][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+                    const u32 hi = (v[b + 1][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+                    out[(c * NB + b) >> 1] = lo | (hi << 16);
+                }
+            }
+            u32x4 *d4 = reinterpret_cast<u32x4 *>(dst + (size_t)8 * i * NB);
+#pragma unroll
+            for (int q = 0; q < NB; ++q) d4[q] = u32x4{out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]};
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const uint16_t *xb = a.x + (size_t)b * (size_t)a.ldx;
-            for (int i = tid; i < nvec; i += BLOCK) {
-                const u32x4 v = reinterpret_cast<const u32x4 *>(xb)[i];
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    dst[(8 * i + e) * NB + b] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
-            }
             for (int i = (nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i * NB + b] = xb[i];
         }
         if (tid < kLdsFront * NB / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
