@@ -82,7 +82,7 @@ int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
 
 /*
  * Y[b, :] = M X[b, :] for b < batch.  X is [batch, ldx] and Y [batch, ldy], row-major fp16 with
- * ldx >= cols and ldy >= rows (elements).  The matrix is streamed once per group of up to four
+ * ldx >= cols and ldy >= rows (elements).  The matrix is streamed once per group of up to eight
  * vectors (as many as fit next to each other in LDS), the rest like macko_spmv_f16.  No
  * counterpart in the upstream package, whose LLM runner maps the single-vector operator over
  * the batch dimension (python_scripts/util_run_pruned_llm.py:112-118).

@@ -120,7 +120,7 @@ def multiply(compressed_M, V):
 
 def multiply_batched(compressed_M, X):
     """Y[b] = M @ X[b] for X of shape (batch, cols) -> (batch, rows).  The matrix is read once per
-    group of up to four vectors.  Upstream has only the single-vector operator and maps it over
+    group of up to eight vectors.  Upstream has only the single-vector operator and maps it over
     the batch dimension (python_scripts/util_run_pruned_llm.py:112-118)."""
     assert compressed_M[0].is_cuda and X.is_cuda
     assert X.dim() == 2 and X.is_contiguous()

@@ -344,7 +344,7 @@ __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
     if (D == 4 && J == 2) MACKO_RING_TAKE("v96", "v97", "v98", "v99", "v106");
     if (D == 4 && J == 3) MACKO_RING_TAKE("v100", "v101", "v102", "v103", "v107");
 }
-// NB = vectors multiplied per launch (1, 2 or 4).  With NB > 1 the NB copies of x are interleaved in
+// NB = vectors multiplied per launch (1, 2, 4 or 8).  With NB > 1 the NB copies of x are interleaved in
 // LDS (element c of vector b at half-word c * NB + b), so one LDS read per stored entry fetches the
 // operand of every vector, and a row ends with NB sums.  NB > 1 exists for fp16 values, x in LDS,
 // plain product only.
@@ -352,10 +352,10 @@ template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
-    static_assert(NB == 1 || (NB <= 4 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
+    static_assert(NB == 1 || (NB <= 8 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int WAVES = BLOCK / kWave;
-    constexpr int kBatchShift = NB == 4 ? 2 : (NB == 2 ? 1 : 0);
+    constexpr int kBatchShift = NB == 8 ? 3 : (NB == 4 ? 2 : (NB == 2 ? 1 : 0));
     constexpr int kTileLoads = 2 * D;  // tracked loads per full ring
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -616,6 +616,7 @@ spmv_stream_kernel(const SpmvArgs a)
     typedef __attribute__((address_space(3))) const uint16_t *lds_u16_ptr;
     typedef __attribute__((address_space(3))) const u32 *lds_u32_ptr;
     typedef __attribute__((address_space(3))) const u32x2 *lds_u32x2_ptr;
+    typedef __attribute__((address_space(3))) const u32x4 *lds_u32x4_ptr;
     // LDS byte address of x[0] (x sits kLdsFront bytes, times NB, into this kernel's dynamic LDS)
     const u32 x_addr = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront * NB;
     // row_addr: LDS byte address the next entry of the current row would read if its nibble were 0,
@@ -636,16 +637,22 @@ spmv_stream_kernel(const SpmvArgs a)
                 const u32 w = vv[k >> 1];
                 const float mv = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
                 const u32 at = x_addr + (addr << kBatchShift) + ((2 * k) << kBatchShift);
+                u32 xs[NB / 2 > 0 ? NB / 2 : 1];  // the NB operands, two per word
                 if (NB == 2) {
-                    const u32 xs = *reinterpret_cast<lds_u32_ptr>(at);
-                    accb[0] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs & 0xffffu)), accb[0]);
-                    accb[1] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs >> 16)), accb[1]);
+                    xs[0] = *reinterpret_cast<lds_u32_ptr>(at);
+                } else if (NB == 4) {
+                    const u32x2 t = *reinterpret_cast<lds_u32x2_ptr>(at);
+                    xs[0] = t.x;
+                    xs[1 % (NB / 2)] = t.y;
                 } else {
-                    const u32x2 xs = *reinterpret_cast<lds_u32x2_ptr>(at);
-                    accb[0] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.x & 0xffffu)), accb[0]);
-                    accb[1] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.x >> 16)), accb[1]);
-                    accb[2 % NB] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.y & 0xffffu)), accb[2 % NB]);
-                    accb[3 % NB] = __builtin_fmaf(mv, half_bits_to_float((uint16_t)(xs.y >> 16)), accb[3 % NB]);
+                    const u32x4 t = *reinterpret_cast<lds_u32x4_ptr>(at);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) xs[q % (NB / 2)] = t[q];
+                }
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const uint16_t h = (b & 1) ? (uint16_t)(xs[b >> 1] >> 16) : (uint16_t)(xs[b >> 1] & 0xffffu);
+                    accb[b] = __builtin_fmaf(mv, half_bits_to_float(h), accb[b]);
                 }
                 continue;
             }
@@ -974,7 +981,7 @@ extern "C" int macko_spmv_i8f16_axpby(const void *values, const void *deltas, co
 }
 
 // Y[b, :] = M X[b, :] for `batch` vectors: X is [batch, ldx] and Y [batch, ldy] row-major fp16
-// (ldx >= cols, ldy >= rows).  The matrix is streamed once per group of up to four vectors (as
+// (ldx >= cols, ldy >= rows).  The matrix is streamed once per group of up to eight vectors (as
 // many as fit in LDS next to each other), so the cost per vector drops accordingly.  The upstream
 // package has no batched entry: its LLM runner maps the single-vector operator over the batch
 // dimension (python_scripts/util_run_pruned_llm.py:112-118).
@@ -1003,7 +1010,10 @@ extern "C" int macko_spmv_f16_batched(const void *values, const void *deltas, co
         a.trace = nullptr;
 #endif
         int step;
-        if (padded_entries > 0 && left >= 4 && 4 * per_vector <= (size_t)info.max_lds_bytes) {
+        if (padded_entries > 0 && left >= 8 && 8 * per_vector <= (size_t)info.max_lds_bytes) {
+            step = 8;
+            rc = spmv_dispatch<false, 2, 8>(a, as_stream(stream));
+        } else if (padded_entries > 0 && left >= 4 && 4 * per_vector <= (size_t)info.max_lds_bytes) {
             step = 4;
             rc = spmv_dispatch<false, 2, 4>(a, as_stream(stream));
         } else if (padded_entries > 0 && left >= 2 && 2 * per_vector <= (size_t)info.max_lds_bytes) {

@@ -250,15 +250,15 @@ def test_multiply_row_lengths_sorted():
                                                (33, 90000, 0.1), (512, 512, 0.0)])
 def test_multiply_batched(rows, cols, density):
     # every vector of the batch against the dense float64 product and against the single-vector path;
-    # batch sizes cover the 4-, 2- and 1-vector launches and their combinations, and LDS limits
-    # (70000 columns: two vectors per launch; 90000: one)
+    # batch sizes cover the 8-, 4-, 2- and 1-vector launches and their combinations, and LDS limits
+    # (20000 columns: four vectors per launch; 70000: two; 90000: one)
     rng = np.random.default_rng(rows + cols)
     dense = helpers.random_sparse(rng, rows, cols, density, scale=0.05)
     if rows > 40:
         dense[3] = 0
         dense[-1] = 0
     compressed = macko_spmv.compress(torch.from_numpy(dense).cuda())
-    for batch in (1, 2, 3, 4, 5, 7, 8):
+    for batch in (1, 2, 3, 4, 5, 7, 8, 9, 15):
         X = rng.standard_normal((batch, cols)).astype(np.float16)
         Xg = torch.from_numpy(X).cuda()
         print("batched case", rows, cols, density, batch, flush=True)
