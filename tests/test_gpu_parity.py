@@ -393,3 +393,27 @@ def test_opcheck_and_compile():
     for _ in range(4):
         out = f_c(V)
         assert torch.allclose((M @ (V + 1)) - 1, out, rtol=1e-3, atol=2e-3)
+
+
+def test_opcheck_of_the_additional_operators():
+    # schema, fake implementation and aliasing annotations of everything beyond the upstream operator
+    torch.manual_seed(1)
+    ops = torch.ops.macko_spmv
+    M = torch.randn((300, 700), dtype=torch.float16, device="cuda")
+    M[torch.rand_like(M.float()) > 0.3] = 0
+    c = macko_spmv.compress(M)
+    V = torch.randn(700, device="cuda", dtype=torch.float16)
+    X = torch.randn(5, 700, device="cuda", dtype=torch.float16)
+    C = torch.randn(300, device="cuda", dtype=torch.float16)
+    torch.library.opcheck(ops.multiply_batched, (*c, X))
+    torch.library.opcheck(ops.multiply_axpby, (*c, V, C, 0.5, 2.0))
+    torch.library.opcheck(ops.decompress, tuple(c))
+    Q = torch.randint(-100, 100, (300, 700), dtype=torch.int8, device="cuda")
+    Q[torch.rand((300, 700), device="cuda") > 0.3] = 0
+    c8 = macko_spmv.compress_int8(Q)
+    torch.library.opcheck(ops.multiply_int8, (*c8, V))
+    torch.library.opcheck(ops.multiply_int8_axpby, (*c8, V, C, 0.5, 2.0))
+    compiled = torch.compile(lambda X: macko_spmv.multiply_batched(c, X * 2), mode="reduce-overhead", fullgraph=True)
+    want = (X.float() * 2) @ M.float().t()
+    for _ in range(3):
+        assert torch.allclose(compiled(X).float(), want, rtol=1e-2, atol=2e-2)
