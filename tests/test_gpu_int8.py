@@ -71,7 +71,7 @@ def _check_product(dense, x, compressed=None):
 
 @pytest.mark.parametrize("shape,density", [((1, 1), 1.0), ((3, 17), 0.5), ((65, 511), 0.3), ((64, 513), 0.9),
                                            ((1000, 1000), 0.05), ((4096, 4096), 0.5), ((11008, 4096), 0.1),
-                                           ((4096, 11008), 0.3), ((37, 30000), 0.2), ((20000, 64), 0.5),
+                                           ((4096, 11008), 0.3), ((37, 30000), 0.2), ((20000, 64), 0.5), ((5, 90000), 0.1),
                                            ((256, 2048), 0.0)])
 def test_multiply_against_dense_float64(shape, density):
     rng = np.random.default_rng(shape[0] * 31 + shape[1])
