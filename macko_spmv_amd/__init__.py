@@ -75,6 +75,18 @@ def _decompress_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols):
     return torch.empty((M_rows, M_cols), device=M_values.device, dtype=M_values.dtype)
 
 
+def _multiply_vmap(info, in_dims, M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
+    """torch.vmap over the vector argument (the way the upstream LLM runner lifts the operator to a
+    sequence of tokens, python_scripts/util_run_pruned_llm.py:109-113) becomes one batched product."""
+    if any(d is not None for d in in_dims[:5]) or in_dims[5] is None:
+        raise NotImplementedError("macko_spmv::multiply: vmap is supported over V only")
+    X = V.movedim(in_dims[5], 0).reshape(info.batch_size, -1).contiguous()
+    return torch.ops.macko_spmv.multiply_batched.default(M_values, M_deltas, M_row_indices, M_rows, M_cols, X), 0
+
+
+torch.library.register_vmap("macko_spmv::multiply", _multiply_vmap)
+
+
 def move_to_device(compressed, device):
     """Move the three tensors of a compressed matrix (src/macko_spmv/__init__.py:110-117)."""
     return (

@@ -417,3 +417,16 @@ def test_opcheck_of_the_additional_operators():
     want = (X.float() * 2) @ M.float().t()
     for _ in range(3):
         assert torch.allclose(compiled(X).float(), want, rtol=1e-2, atol=2e-2)
+
+
+def test_vmap_over_the_vector_like_the_upstream_llm_layer():
+    # python_scripts/util_run_pruned_llm.py:109-118: torch.vmap(f, in_dims=-2, out_dims=-2) over (1, t, C)
+    torch.manual_seed(2)
+    M = torch.randn((300, 700), dtype=torch.float16, device="cuda")
+    M[torch.rand_like(M.float()) > 0.3] = 0
+    c = macko_spmv.compress(M)
+    lifted = torch.vmap(lambda x: macko_spmv.multiply(c, x), in_dims=-2, out_dims=-2)
+    x = torch.randn(1, 6, 700, device="cuda", dtype=torch.float16)
+    out = lifted(x)
+    assert out.shape == (6, 300)
+    assert torch.allclose(out.float(), x[0].float() @ M.float().t(), rtol=1e-2, atol=2e-2)
