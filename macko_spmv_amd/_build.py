@@ -73,8 +73,11 @@ FIXED_VGPR_BASE = 78
 
 
 def verify_fixed_registers(verbose=False):
-    """Compile macko_spmv.hip to assembly and check that, outside the hand-written asm blocks, no
-    instruction of any spmv_stream_kernel touches a VGPR >= FIXED_VGPR_BASE."""
+    """Compile macko_spmv.hip to assembly and check two things the hand-tracked loads of every
+    spmv_stream_kernel rely on: outside the hand-written asm blocks no instruction touches a VGPR
+    >= FIXED_VGPR_BASE, and the compiler has put no vmcnt wait of its own right in front of a ring
+    take (it does when one of its own loads may still be outstanding at the loop's back edge; such
+    a wait also waits for the ring loads in flight and serialises the stream)."""
     with tempfile.TemporaryDirectory() as tmp:
         asm = os.path.join(tmp, "macko_spmv.s")
         _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, "macko_spmv.hip"), "-o", asm],
@@ -83,22 +86,32 @@ def verify_fixed_registers(verbose=False):
     kernel = None
     in_asm = False
     checked = 0
-    for line in text:
+    recent_wait = None  # (line number, text) of the last compiler-generated vmcnt wait
+    for number, line in enumerate(text):
         m = re.match(r"^(_Z\S*spmv_stream_kernel\S*):", line)
         if m:
-            kernel, in_asm = m.group(1), False
+            kernel, in_asm, recent_wait = m.group(1), False, None
             checked += 1
             continue
         if kernel is None:
             continue
-        if "s_endpgm" in line:
+        if line.startswith(".Lfunc_end") or ".amdhsa_kernel" in line:
             kernel = None
         elif "#ASMSTART" in line:
             in_asm = True
         elif "#ASMEND" in line:
             in_asm = False
-        elif not in_asm:
+        elif in_asm:
+            # a ring take copies out of v88.. after its own wait
+            if recent_wait and number - recent_wait[0] <= 16 and re.search(r"v_mov_b32 \S+ v(88|92|96|100)\b", line):
+                raise RuntimeError(f"compiler-generated '{recent_wait[1]}' in front of a ring take in {kernel} "
+                                   f"(assembly line {recent_wait[0] + 1})")
+        else:
             code = line.split(";")[0]
+            if re.match(r"^\s*\.L?BB\d+_\d+:", code):
+                recent_wait = None  # a label: what follows is another block
+            if re.search(r"s_waitcnt\b.*vmcnt\(", code):
+                recent_wait = (number, code.strip())
             regs = [int(b) for _, b in re.findall(r"\bv\[(\d+):(\d+)\]", code)]
             regs += [int(a) for a in re.findall(r"\bv(\d+)\b", code)]
             if regs and max(regs) >= FIXED_VGPR_BASE:

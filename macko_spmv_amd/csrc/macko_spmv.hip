@@ -470,6 +470,10 @@ spmv_stream_kernel(const SpmvArgs a)
         if (__builtin_expect(r < win_base || r + 1 > win_base + 63, 0)) {
             win_base = r;
             win = load_row_window(a.row_ptr, a.rows, win_base, lane);
+            // Awaited on the spot: a load the compiler still counts as outstanding at the loop's
+            // back edge makes it protect the register with a vmcnt(0) at the top of every
+            // iteration, which would also wait for the ring loads just issued.
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), expcnt and lgkmcnt untouched
         }
     };
     auto store_row = [&](int r, float total, int b = 0) {
@@ -574,6 +578,9 @@ spmv_stream_kernel(const SpmvArgs a)
                 s_end = row_last >= win_base && row_last <= win_base + 63 ? row_start(row_last)
                                                                             : uniform(a.row_ptr[row_last]);
         }
+        // nothing the compiler loaded on this path may still count as outstanding when the tile
+        // loop is entered (see slide_window)
+        __builtin_amdgcn_s_waitcnt(0x0f70);
     }
 
     // ---- 4. my tile range; the ring is filled with my first D tiles before x is even in LDS: they
@@ -852,7 +859,9 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     // start, when a wave owns a single row or only a few tiles; waves that walk many tiles over
     // several rows do slightly better with two (measured on the Llama shapes; deeper is slower).
     const long long n_waves = grid * waves;
-    const int depth = t.depth ? t.depth : ((long long)a.rows > n_waves && n_tiles >= 6 * n_waves ? 2 : 1);
+    // The int8 variant, bound by its arithmetic rather than by memory, takes two whenever the walk is long.
+    const bool long_walk = n_tiles >= 6 * n_waves;
+    const int depth = t.depth ? t.depth : (long_walk && (VB == 1 || (long long)a.rows > n_waves) ? 2 : 1);
 
     const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack);
     if (NB > 1) {  // NB vectors per launch: the caller has checked that they fit in LDS
