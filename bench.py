@@ -36,7 +36,7 @@ LARGE_DENSITIES = [0.1, 0.3, 0.5]
 # default workload: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, each scaled by what the
 # same counter reports for calibration_copy_kernel on 256 MiB (factors 0.5000 and 1.0000).  Source:
 # profiles/spmv_stream_kernel_llama_shapes_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 42.82e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 42.81e6}
 
 WORKLOADS = {
     "llama": "configs[1]: Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as fp16 SpMV, per-row "
