@@ -72,17 +72,13 @@ _DEVICE_FLAGS = [
 FIXED_VGPR_BASE = 78
 
 
-def verify_fixed_registers(verbose=False):
-    """Compile macko_spmv.hip to assembly and check two things the hand-tracked loads of every
-    spmv_stream_kernel rely on: outside the hand-written asm blocks no instruction touches a VGPR
-    >= FIXED_VGPR_BASE, and the compiler has put no vmcnt wait of its own right in front of a ring
-    take (it does when one of its own loads may still be outstanding at the loop's back edge; such
-    a wait also waits for the ring loads in flight and serialises the stream)."""
-    with tempfile.TemporaryDirectory() as tmp:
-        asm = os.path.join(tmp, "macko_spmv.s")
-        _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, "macko_spmv.hip"), "-o", asm],
-             verbose)
-        text = open(asm).read().splitlines()
+def check_stream_kernel_assembly(text):
+    """`text`: lines of the assembly of macko_spmv.hip.  Checks two things the hand-tracked loads of
+    every spmv_stream_kernel rely on: outside the hand-written asm blocks no instruction touches a
+    VGPR >= FIXED_VGPR_BASE, and the compiler has put no vmcnt wait of its own right in front of a
+    ring take (it does when one of its own loads may still be outstanding at the loop's back edge;
+    such a wait also waits for the ring loads in flight and serialises the stream).  Returns the
+    number of kernels checked; raises RuntimeError on a violation."""
     kernel = None
     in_asm = False
     checked = 0
@@ -119,6 +115,16 @@ def verify_fixed_registers(verbose=False):
     if checked == 0:
         raise RuntimeError("no spmv_stream_kernel found in the assembly; the register check is stale")
     return checked
+
+
+def verify_fixed_registers(verbose=False):
+    """Compile macko_spmv.hip to assembly and run check_stream_kernel_assembly on it."""
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "macko_spmv.s")
+        _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, "macko_spmv.hip"), "-o", asm],
+             verbose)
+        text = open(asm).read().splitlines()
+    return check_stream_kernel_assembly(text)
 
 
 def build_hip(verbose=False):

@@ -129,3 +129,29 @@ def test_product_package_does_not_touch_the_oracle():
             if name.endswith((".py", ".hip", ".cpp", ".h")):
                 text = open(os.path.join(dirpath, name)).read()
                 assert "oracle" not in text, f"{name} mentions the oracle"
+
+
+def test_assembly_check_of_the_hand_tracked_loads():
+    # the build refuses assembly in which compiler-generated code would break the stream kernel's
+    # hand-counted waits; exercised here on synthetic listings
+    from macko_spmv_amd import _build
+
+    head = ["_ZN5macko12_GLOBAL__N_118spmv_stream_kernelILi1024ELi2ELb1ELb0ELi2ELi1EEEvNS0_8SpmvArgsE: ; @x"]
+    take = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(2)", "\tv_mov_b32 v0, v88", "\t;;#ASMEND"]
+    tail = ["\ts_endpgm", ".Lfunc_end0:"]
+    clean = head + ["\ts_barrier", ".LBB0_1:", "\tv_add_u32_e32 v4, s2, v8"] + take + ["\tv_fma_f32 v5, v0, v1, v5"] + tail
+    assert _build.check_stream_kernel_assembly(clean) == 1
+    # code behind an early s_endpgm still belongs to the kernel
+    late = head + ["\ts_endpgm", ".LBB0_9:", "\tv_mov_b32_e32 v90, 0"] + tail
+    with pytest.raises(RuntimeError, match="fixed VGPR"):
+        _build.check_stream_kernel_assembly(late)
+    with pytest.raises(RuntimeError, match="fixed VGPR"):
+        _build.check_stream_kernel_assembly(head + ["\tglobal_load_dwordx4 v[76:79], v[2:3], off"] + tail)
+    waiting = head + [".LBB0_1:", "\ts_waitcnt vmcnt(0)", "\tv_or_b32_e32 v4, s2, v8"] + take + tail
+    with pytest.raises(RuntimeError, match="in front of a ring take"):
+        _build.check_stream_kernel_assembly(waiting)
+    # a wait in another block (behind a label) or one that does not touch vmcnt is fine
+    assert _build.check_stream_kernel_assembly(
+        head + ["\ts_waitcnt vmcnt(0)", ".LBB0_2:", "\ts_waitcnt lgkmcnt(0)"] + take + tail) == 1
+    with pytest.raises(RuntimeError, match="stale"):
+        _build.check_stream_kernel_assembly(["\ts_nop 0"])
