@@ -42,6 +42,17 @@ int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v
                                const int64_t *position, void *out, int32_t n_heads,
                                int32_t head_dim, int32_t max_len, float scale, void *stream);
 
+/*
+ * macko_decode_rope_append_f16 followed by macko_decode_attention_f16 in one launch: q, k, v are
+ * the raw projections of the current token, the caches receive the rotated k and v at *position,
+ * out is the attention output.  Same limits as the two separate calls.
+ */
+int macko_decode_rope_attention_f16(const void *q, const void *k, const void *v,
+                                    const float *cos_table, const float *sin_table,
+                                    const int64_t *position, void *k_cache, void *v_cache,
+                                    void *out, int32_t n_heads, int32_t head_dim, int32_t max_len,
+                                    float scale, void *stream);
+
 /* out[i] = silu(gate[i]) * up[i], i < n. */
 int macko_decode_silu_mul_f16(const void *gate, const void *up, void *out, int32_t n,
                               void *stream);

@@ -93,6 +93,25 @@ int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t
                            void *stream);
 
 /*
+ * Products whose input vector is produced on the fly while it is staged for the product, so a
+ * decode step needs no launch for the producer.  No counterpart in the upstream package, whose
+ * LLM runner leaves these parts to stock modules (python_scripts/util_run_pruned_llm.py:136-160).
+ * Both need cols % 8 == 0, 16-byte aligned vector operands, and a vector that fits in LDS
+ * (cols <= 81,000 or so); MACKO_E_INVALID_ARGUMENT otherwise.
+ *
+ * macko_spmv_f16_rmsnorm:        y = M n,  n[i] = fp16(x[i] * rsqrt(mean(x^2) + eps) * norm_weight[i])
+ * macko_spmv_f16_silu_mul_axpby: y = alpha * M g + beta * y,  g[i] = fp16(silu(gate[i]) * up[i]);
+ *                                with alpha == 1 and beta == 0, y is not read.
+ */
+int macko_spmv_f16_rmsnorm(const void *values, const void *deltas, const int32_t *row_ptr,
+                           const void *x, const void *norm_weight, float eps, void *y,
+                           int32_t rows, int32_t cols, int64_t padded_entries, void *stream);
+int macko_spmv_f16_silu_mul_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+                                  const void *gate, const void *up, void *y, int32_t rows,
+                                  int32_t cols, int64_t padded_entries, float alpha, float beta,
+                                  void *stream);
+
+/*
  * int8 values variant.  Same arrays, except that `values` holds int8 [P] (8-byte aligned) and
  * `dense` is a row-major int8 matrix.  The compressor pair replaces compress_rows_int8_cpu
  * (src/macko_spmv/cuda/cpu_compressor.cuh:75-117), which differs from the fp16 one in keeping

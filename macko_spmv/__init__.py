@@ -12,4 +12,6 @@ from macko_spmv_amd import (  # noqa: F401
     multiply_batched,
     multiply_int8,
     multiply_int8_axpby,
+    multiply_rmsnorm,
+    multiply_silu_mul_axpby,
 )

@@ -60,6 +60,21 @@ def _multiply_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C
     return None
 
 
+@torch.library.register_fake("macko_spmv::multiply_rmsnorm")
+def _multiply_rmsnorm_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, norm_weight, eps):
+    return torch.empty((M_rows,), device=M_values.device, dtype=M_values.dtype)
+
+
+@torch.library.register_fake("macko_spmv::multiply_silu_mul_axpby")
+def _multiply_silu_mul_axpby_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, gate, up, C, alpha, beta):
+    return None
+
+
+@torch.library.register_fake("macko_spmv::decode_rope_attention")
+def _decode_rope_attention_fake(q, k, v, cos_table, sin_table, position, k_cache, v_cache, scale):
+    return torch.empty_like(q)
+
+
 @torch.library.register_fake("macko_spmv::multiply_int8")
 def _multiply_int8_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
     return torch.empty((M_rows,), device=V.device, dtype=V.dtype)
@@ -148,6 +163,22 @@ def multiply_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):
         compressed_M[0], compressed_M[1], compressed_M[2], compressed_M[3], compressed_M[4], V, C,
         float(alpha), float(beta),
     )
+    return C
+
+
+def multiply_rmsnorm(compressed_M, V, norm_weight, eps):
+    """M @ rmsnorm(V) with rmsnorm(V) = fp16(V * rsqrt(mean(V^2) + eps) * norm_weight), the norm
+    applied while the product stages its input (no launch, no round trip through memory for it).
+    Needs cols % 8 == 0 and a vector that fits in LDS.  No upstream counterpart."""
+    assert compressed_M[0].is_cuda and V.is_cuda and norm_weight.is_cuda
+    return torch.ops.macko_spmv.multiply_rmsnorm.default(*compressed_M[:5], V, norm_weight, float(eps))
+
+
+def multiply_silu_mul_axpby(compressed_M, gate, up, C, alpha=1.0, beta=0.0):
+    """In place C = alpha * M @ (silu(gate) * up) + beta * C: the gated activation of a Llama MLP
+    applied while the down projection stages its input.  Same limits as multiply_rmsnorm."""
+    assert compressed_M[0].is_cuda and gate.is_cuda and up.is_cuda and C.is_cuda
+    torch.ops.macko_spmv.multiply_silu_mul_axpby.default(*compressed_M[:5], gate, up, C, float(alpha), float(beta))
     return C
 
 

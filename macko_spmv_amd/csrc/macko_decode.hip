@@ -82,11 +82,18 @@ __global__ void rope_append_kernel(const uint16_t *__restrict__ q, const uint16_
 
 // Single-query attention over positions 0..position of one head per workgroup (256 threads):
 // scores, softmax, weighted sum of v.  head_dim <= 256 and a multiple of 8; max_len <= kMaxLen.
+// With ROPE the kernel first does what rope_append_kernel does for its head (q, k, v are then the
+// raw projections; the rotated q is rounded to fp16 as if it had been written out), so a decode
+// step needs one launch for both.
 constexpr int kAttnThreads = 256;
 constexpr int kMaxLen = 4096;
+template <bool ROPE>
 __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t *__restrict__ q,
-                                                                  const uint16_t *__restrict__ k_cache,
-                                                                  const uint16_t *__restrict__ v_cache,
+                                                                  const uint16_t *__restrict__ k_new,
+                                                                  const uint16_t *__restrict__ v_new,
+                                                                  const float *__restrict__ cos_table,
+                                                                  const float *__restrict__ sin_table,
+                                                                  uint16_t *k_cache, uint16_t *v_cache,
                                                                   const long long *__restrict__ position,
                                                                   uint16_t *__restrict__ out, int head_dim, int max_len,
                                                                   float scale)
@@ -99,7 +106,26 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
     long long pos = position[0];
     pos = pos < 0 ? 0 : (pos >= max_len ? max_len - 1 : pos);
     const int len = (int)pos + 1;
-    if (tid < head_dim) qs[tid] = h2f(q[(size_t)head * head_dim + tid]) * scale;
+    if (ROPE) {
+        const int half = head_dim >> 1;
+        if (tid < half) {
+            const int i = tid;
+            const float c = cos_table[pos * half + i], s = sin_table[pos * half + i];
+            const size_t in = (size_t)head * head_dim;
+            const size_t slot = ((size_t)head * max_len + (size_t)pos) * head_dim;
+            const float q0 = h2f(q[in + i]), q1 = h2f(q[in + i + half]);
+            qs[i] = h2f(f2h(q0 * c - q1 * s)) * scale;
+            qs[i + half] = h2f(f2h(q1 * c + q0 * s)) * scale;
+            const float k0 = h2f(k_new[in + i]), k1 = h2f(k_new[in + i + half]);
+            k_cache[slot + i] = f2h(k0 * c - k1 * s);
+            k_cache[slot + i + half] = f2h(k1 * c + k0 * s);
+            v_cache[slot + i] = v_new[in + i];
+            v_cache[slot + i + half] = v_new[in + i + half];
+        }
+        __threadfence();  // the new cache row is read back below by other threads of this workgroup
+    } else if (tid < head_dim) {
+        qs[tid] = h2f(q[(size_t)head * head_dim + tid]) * scale;
+    }
     __syncthreads();
     const uint16_t *kh = k_cache + (size_t)head * max_len * head_dim;
     const uint16_t *vh = v_cache + (size_t)head * max_len * head_dim;
@@ -203,9 +229,30 @@ extern "C" int macko_decode_attention_f16(const void *q, const void *k_cache, co
         return MACKO_E_INVALID_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(k_cache) & 15) || (reinterpret_cast<uintptr_t>(v_cache) & 15))
         return MACKO_E_INVALID_ARGUMENT;
-    hipLaunchKernelGGL(attention_kernel, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
-                       (const uint16_t *)q, (const uint16_t *)k_cache, (const uint16_t *)v_cache,
-                       (const long long *)position, (uint16_t *)out, head_dim, max_len, scale);
+    hipLaunchKernelGGL(attention_kernel<false>, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
+                       (const uint16_t *)q, (const uint16_t *)nullptr, (const uint16_t *)nullptr,
+                       (const float *)nullptr, (const float *)nullptr, (uint16_t *)const_cast<void *>(k_cache),
+                       (uint16_t *)const_cast<void *>(v_cache), (const long long *)position, (uint16_t *)out,
+                       head_dim, max_len, scale);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_decode_rope_attention_f16(const void *q, const void *k, const void *v, const float *cos_table,
+                                               const float *sin_table, const int64_t *position, void *k_cache,
+                                               void *v_cache, void *out, int32_t n_heads, int32_t head_dim,
+                                               int32_t max_len, float scale, void *stream)
+{
+    using namespace macko;
+    if (!q || !k || !v || !cos_table || !sin_table || !position || !k_cache || !v_cache || !out)
+        return MACKO_E_INVALID_ARGUMENT;
+    if (n_heads <= 0 || head_dim <= 0 || head_dim > 256 || (head_dim & 7) || max_len <= 0 || max_len > kMaxLen)
+        return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(k_cache) & 15) || (reinterpret_cast<uintptr_t>(v_cache) & 15))
+        return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(attention_kernel<true>, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
+                       (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, cos_table, sin_table,
+                       (uint16_t *)k_cache, (uint16_t *)v_cache, (const long long *)position, (uint16_t *)out,
+                       head_dim, max_len, scale);
     return (int)hipGetLastError();
 }
 

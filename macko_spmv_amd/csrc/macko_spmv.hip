@@ -52,6 +52,9 @@ struct SpmvArgs {
     u32 row_even;
     // batched product (NB > 1 vectors per launch): elements between consecutive vectors of x / y
     int ldx, ldy;
+    // fused x staging (XF != 0): the second operand of the function that produces x, and its epsilon
+    const uint16_t *x2;
+    float eps;
 #ifdef MACKO_SPMV_TRACE
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif
@@ -348,11 +351,16 @@ __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
 // LDS (element c of vector b at half-word c * NB + b), so one LDS read per stored entry fetches the
 // operand of every vector, and a row ends with NB sums.  NB > 1 exists for fp16 values, x in LDS,
 // plain product only.
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB>
+// XF = function applied to the input while it is staged into LDS, so the producer of x needs no
+// launch of its own: 0 = none (x as given), 1 = RMS norm (x * rsqrt(mean(x^2) + eps) * x2, x2 the
+// norm weight), 2 = SiLU gate (silu(x) * x2).  The staged vector is rounded to fp16 exactly as a
+// separate kernel writing it to memory would.  XF != 0 needs cols % 8 == 0 and 16-byte aligned x, x2.
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB, int XF>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
     static_assert(NB == 1 || (NB <= 8 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
+    static_assert(XF == 0 || (NB == 1 && X_LDS && VB == 2), "fused staging: fp16, one vector, x in LDS");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int WAVES = BLOCK / kWave;
     constexpr int kBatchShift = NB == 8 ? 3 : (NB == 4 ? 2 : (NB == 2 ? 1 : 0));
@@ -398,7 +406,7 @@ spmv_stream_kernel(const SpmvArgs a)
         probe_issue<1>((u32)i1 * 4, buf_rows);
     }
     const u32x4 buf_x = make_buffer(a.x, (u32)x_nvec * 16);  // past the end reads as zero
-    if (X_LDS && NB == 1) {
+    if (X_LDS && NB == 1 && XF == 0) {
         xpiece_issue<0>((u32)tid * 16, buf_x);
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
@@ -443,6 +451,52 @@ spmv_stream_kernel(const SpmvArgs a)
         }
         if (tid < kLdsFront * NB / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
         if (tid < kLdsBack * NB / 2) dst[a.cols * NB + tid] = 0;
+    } else if (XF != 0) {
+        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
+        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
+        const int nvec = a.cols >> 3;
+        auto lo = [](u32 w) { return half_bits_to_float((uint16_t)(w & 0xffffu)); };
+        auto hi = [](u32 w) { return half_bits_to_float((uint16_t)(w >> 16)); };
+        auto pack = [](float l, float h) { return (u32)float_to_half_bits(l) | ((u32)float_to_half_bits(h) << 16); };
+        if (XF == 1) {
+            // pass 1: raw x into LDS and the sum of squares; pass 2: each thread scales the pieces
+            // it wrote itself, so only the sum needs a barrier
+            float ss = 0.f;
+            for (int i = tid; i < nvec; i += BLOCK) {
+                const u32x4 v = reinterpret_cast<const u32x4 *>(a.x)[i];
+                d4[i] = v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ss += lo(v[e]) * lo(v[e]) + hi(v[e]) * hi(v[e]);
+            }
+            float *red = reinterpret_cast<float *>(lds + kLdsFront + 2 * (size_t)a.cols + kLdsBack);
+            const float ws = wave_sum(ss);
+            if (lane == 0) red[wave] = ws;
+            __syncthreads();
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) total += red[w];
+            const float inv = rsqrtf(total / (float)a.cols + a.eps);
+            for (int i = tid; i < nvec; i += BLOCK) {
+                const u32x4 v = d4[i];
+                const u32x4 g = reinterpret_cast<const u32x4 *>(a.x2)[i];
+                u32x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = pack(lo(v[e]) * inv * lo(g[e]), hi(v[e]) * inv * hi(g[e]));
+                d4[i] = o;
+            }
+        } else {
+            auto gate = [](float g, float u) { return g / (1.0f + __expf(-g)) * u; };
+            for (int i = tid; i < nvec; i += BLOCK) {
+                const u32x4 g = reinterpret_cast<const u32x4 *>(a.x)[i];
+                const u32x4 u = reinterpret_cast<const u32x4 *>(a.x2)[i];
+                u32x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = pack(gate(lo(g[e]), lo(u[e])), gate(hi(g[e]), hi(u[e])));
+                d4[i] = o;
+            }
+        }
+        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
+        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
     } else if (X_LDS) {
         uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
         u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
@@ -456,7 +510,7 @@ spmv_stream_kernel(const SpmvArgs a)
     MACKO_STAMP(1);
 
     // ---- 3. which rows are mine -----------------------------------------------------------------------
-    constexpr int kXLoads = X_LDS && NB == 1 ? kXRegs : 0;
+    constexpr int kXLoads = X_LDS && NB == 1 && XF == 0 ? kXRegs : 0;
     int window[2];
     window[0] = probe_take<0, kXLoads + 1>();
     window[1] = probe_take<1, kXLoads>();
@@ -596,7 +650,7 @@ spmv_stream_kernel(const SpmvArgs a)
     }
 
     // ---- 5. x pieces into LDS (older than the ring loads just issued, if any) ---------------------------
-    if (NB > 1) {
+    if (NB > 1 || XF != 0) {
         __syncthreads();
     } else if (X_LDS) {
         const u32 lds_x = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
@@ -794,10 +848,10 @@ __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1>
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1, int XF = 0>
 int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB>;
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
     a.entries_q = (u32)(a.padded / n_waves);
     a.entries_rem = (u32)(a.padded % n_waves);
@@ -829,7 +883,7 @@ struct Tuning {
 };
 Tuning g_tuning = {0, 0, 0};
 
-template <bool AXPBY, int VB = 2, int NB = 1>
+template <bool AXPBY, int VB = 2, int NB = 1, int XF = 0>
 int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
 {
     if (a.rows == 0) return 0;
@@ -863,7 +917,12 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     const bool long_walk = n_tiles >= 6 * n_waves;
     const int depth = t.depth ? t.depth : (long_walk && (VB == 1 || (long long)a.rows > n_waves) ? 2 : 1);
 
-    const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack);
+    const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack) + (XF == 1 ? 64 : 0);
+    if (XF != 0) {  // fused staging: x must fit in LDS (checked by the caller too)
+        if (lds_need > (size_t)info.max_lds_bytes || block != 1024) return MACKO_E_INVALID_ARGUMENT;
+        if (depth == 2) return launch_stream<1024, 2, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_need, stream);
+        return launch_stream<1024, 1, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_need, stream);
+    }
     if (NB > 1) {  // NB vectors per launch: the caller has checked that they fit in LDS
         if (lds_need > (size_t)info.max_lds_bytes || block != 1024) return MACKO_E_INVALID_ARGUMENT;
         if (depth == 2) return launch_stream<1024, 2, true, false, 2, NB>(a, (int)grid, lds_need, stream);
@@ -1036,4 +1095,63 @@ extern "C" int macko_spmv_f16_batched(const void *values, const void *deltas, co
         done += step;
     }
     return 0;
+}
+
+namespace macko {
+namespace {
+// Extra conditions of the fused-input variants: whole 16-byte pieces only, and x must fit in LDS.
+int check_fused_args(const void *x, const void *x2, int32_t cols, int64_t padded)
+{
+    if (padded == 0) return 0;
+    if (x2 == nullptr || (cols & 7) != 0) return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(x2) & 15)) return MACKO_E_INVALID_ARGUMENT;
+    DeviceInfo info;
+    int rc = device_info(&info);
+    if (rc != 0) return rc;
+    if ((size_t)kLdsFront + 2 * (size_t)cols + kLdsBack + 64 > (size_t)info.max_lds_bytes) return MACKO_E_INVALID_ARGUMENT;
+    return 0;
+}
+}  // namespace
+}  // namespace macko
+
+// y = M * rmsnorm(x), rmsnorm(x)[i] = fp16(x[i] * rsqrt(mean(x^2) + eps) * norm_weight[i]): the
+// normalisation in front of a projection, folded into the product's own staging of its input.
+// No upstream counterpart: the upstream harness runs the stock module for the norm
+// (python_scripts/util_run_pruned_llm.py:136-160).
+extern "C" int macko_spmv_f16_rmsnorm(const void *values, const void *deltas, const int32_t *row_ptr, const void *x,
+                                      const void *norm_weight, float eps, void *y, int32_t rows, int32_t cols,
+                                      int64_t padded_entries, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
+    if (rc != 0) return rc;
+    rc = check_fused_args(x, norm_weight, cols, padded_entries);
+    if (rc != 0) return rc;
+    SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
+               rows, cols, padded_entries, 1.0f, 0.0f, 0, 0, 0, 0, 0, 0, 0, (const uint16_t *)norm_weight, eps};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = nullptr;
+#endif
+    return spmv_dispatch<false, 2, 1, 1>(a, as_stream(stream));
+}
+
+// y = alpha * M * (silu(gate) .* up) + beta * y: the gated activation of a Llama MLP folded into
+// the down projection's staging of its input, and the residual into its epilogue.  alpha == 1
+// with beta == 0 leaves y unread.  No upstream counterpart (see above).
+extern "C" int macko_spmv_f16_silu_mul_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+                                             const void *gate, const void *up, void *y, int32_t rows, int32_t cols,
+                                             int64_t padded_entries, float alpha, float beta, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, gate, y, rows, cols, padded_entries);
+    if (rc != 0) return rc;
+    rc = check_fused_args(gate, up, cols, padded_entries);
+    if (rc != 0) return rc;
+    SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)gate, (uint16_t *)y,
+               rows, cols, padded_entries, alpha, beta, 0, 0, 0, 0, 0, 0, 0, (const uint16_t *)up, 0.0f};
+#ifdef MACKO_SPMV_TRACE
+    a.trace = nullptr;
+#endif
+    if (beta == 0.0f && alpha == 1.0f) return spmv_dispatch<false, 2, 1, 2>(a, as_stream(stream));
+    return spmv_dispatch<true, 2, 1, 2>(a, as_stream(stream));
 }

@@ -320,6 +320,88 @@ at::Tensor decode_silu_mul_hip(const at::Tensor &gate, const at::Tensor &up)
     return out;
 }
 
+void check_macko_operands(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                          int64_t M_rows, int64_t M_cols)
+{
+    TORCH_CHECK(M_values.dtype() == at::kHalf && M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt,
+                "bad matrix dtypes");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda(), "the matrix must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
+                "the matrix tensors must be contiguous");
+    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
+    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
+    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+}
+
+// M @ rmsnorm(V): the norm is applied while V is staged for the product.
+at::Tensor multiply_rmsnorm_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                                const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &V,
+                                const at::Tensor &norm_weight, double eps)
+{
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(V, "V");
+    check_half_gpu(norm_weight, "norm_weight");
+    TORCH_CHECK(V.numel() == M_cols && norm_weight.numel() == M_cols, "V and norm_weight must hold M_cols elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    at::Tensor C = at::empty({M_rows}, M_values.options());
+    check_rc(macko_spmv_f16_rmsnorm(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                    V.data_ptr(), norm_weight.data_ptr(), (float)eps, C.data_ptr(), (int32_t)M_rows,
+                                    (int32_t)M_cols, M_values.numel(),
+                                    (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "multiply_rmsnorm");
+    return C;
+}
+
+// C = alpha * M @ (silu(gate) * up) + beta * C, in place on C.
+void multiply_silu_mul_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                                 const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols,
+                                 const at::Tensor &gate, const at::Tensor &up, at::Tensor C, double alpha, double beta)
+{
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(gate, "gate");
+    check_half_gpu(up, "up");
+    check_half_gpu(C, "C");
+    TORCH_CHECK(gate.numel() == M_cols && up.numel() == M_cols, "gate and up must hold M_cols elements");
+    TORCH_CHECK(C.numel() >= M_rows, "C must hold M_rows elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    check_rc(macko_spmv_f16_silu_mul_axpby(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                           gate.data_ptr(), up.data_ptr(), C.data_ptr(), (int32_t)M_rows,
+                                           (int32_t)M_cols, M_values.numel(), (float)alpha, (float)beta,
+                                           (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "multiply_silu_mul_axpby");
+}
+
+// Rotary embedding, cache append and attention of one decode step in one launch; q, k, v are the
+// raw projections.  Returns the attention output [n_heads * head_dim].
+at::Tensor decode_rope_attention_hip(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
+                                     const at::Tensor &cos_table, const at::Tensor &sin_table,
+                                     const at::Tensor &position, at::Tensor k_cache, at::Tensor v_cache, double scale)
+{
+    check_half_gpu(q, "q");
+    check_half_gpu(k, "k");
+    check_half_gpu(v, "v");
+    check_half_gpu(k_cache, "k_cache");
+    check_half_gpu(v_cache, "v_cache");
+    TORCH_CHECK(k_cache.dim() == 3 && v_cache.sizes() == k_cache.sizes(), "caches must be [heads, max_len, head_dim]");
+    const int64_t n_heads = k_cache.size(0), max_len = k_cache.size(1), head_dim = k_cache.size(2);
+    TORCH_CHECK(q.numel() == n_heads * head_dim && k.numel() == q.numel() && v.numel() == q.numel(), "bad q/k/v size");
+    TORCH_CHECK(cos_table.is_cuda() && cos_table.dtype() == at::kFloat && cos_table.is_contiguous() &&
+                    cos_table.numel() == max_len * (head_dim / 2) && sin_table.is_cuda() &&
+                    sin_table.dtype() == at::kFloat && sin_table.is_contiguous() &&
+                    sin_table.numel() == cos_table.numel(),
+                "cos/sin tables must be contiguous float32 GPU tensors [max_len, head_dim/2]");
+    TORCH_CHECK(position.is_cuda() && position.dtype() == at::kLong && position.numel() == 1, "bad position");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+    at::Tensor out = at::empty_like(q);
+    check_rc(macko_decode_rope_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos_table.data_ptr<float>(),
+                                             sin_table.data_ptr<float>(), position.data_ptr<int64_t>(),
+                                             k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), (int32_t)n_heads,
+                                             (int32_t)head_dim, (int32_t)max_len, (float)scale,
+                                             (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
+             "decode_rope_attention");
+    return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(macko_spmv, m)
@@ -341,6 +423,12 @@ TORCH_LIBRARY(macko_spmv, m)
           "Tensor(a!) k_cache, Tensor(b!) v_cache) -> Tensor");
     m.def("decode_attention(Tensor q, Tensor k_cache, Tensor v_cache, Tensor position, float scale) -> Tensor");
     m.def("decode_silu_mul(Tensor gate, Tensor up) -> Tensor");
+    m.def("multiply_rmsnorm(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V, Tensor norm_weight, float eps) -> Tensor");
+    m.def("multiply_silu_mul_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor gate, Tensor up, Tensor(a!) C, float alpha, float beta) -> ()");
+    m.def("decode_rope_attention(Tensor q, Tensor k, Tensor v, Tensor cos_table, Tensor sin_table, Tensor position, "
+          "Tensor(a!) k_cache, Tensor(b!) v_cache, float scale) -> Tensor");
     m.def("decompress(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols) -> Tensor");
 }
 
@@ -357,6 +445,9 @@ TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
     m.impl("decode_rope_append", &decode_rope_append_hip);
     m.impl("decode_attention", &decode_attention_hip);
     m.impl("decode_silu_mul", &decode_silu_mul_hip);
+    m.impl("multiply_rmsnorm", &multiply_rmsnorm_hip);
+    m.impl("multiply_silu_mul_axpby", &multiply_silu_mul_axpby_hip);
+    m.impl("decode_rope_attention", &decode_rope_attention_hip);
     m.impl("decompress", &decompress_hip);
 }
 

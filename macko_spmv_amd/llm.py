@@ -274,11 +274,18 @@ class DecodeEngine:
     (y = Mx + y), and the parts between the products (RMSNorm, rotary + KV-cache append, attention,
     SiLU * up) as one hand-written kernel each.  Works on a LlamaDecoder whose projections are either
     nn.Linear (dense) or MackoLinear; the model's projection modules are consumed (set to None) so
-    the weights are held once."""
+    the weights are held once.
 
-    def __init__(self, model):
+    With fuse=True (the default) a step drops to five launches per layer: rotary, cache append and
+    attention share one kernel, and, for MACKO projections, the two RMS norms and the SiLU gate are
+    applied by the product that consumes them while it stages its input (multiply_rmsnorm,
+    multiply_silu_mul_axpby).  Dense projections go through the BLAS matrix-vector product, which
+    has no such hook, and keep their separate norm and gate kernels."""
+
+    def __init__(self, model, fuse=True):
         ops = torch.ops.macko_spmv
         self.ops = ops
+        self.fuse = fuse
         body = model.model
         first = body.layers[0].self_attn
         self.n_heads, self.head_dim, self.max_len = first.n_heads, first.head_dim, first.max_len
@@ -349,15 +356,25 @@ class DecodeEngine:
         ops, H, I = self.ops, self.dim, self.hidden
         x = self.embed.index_select(0, token).view(-1)
         for L in self.layers:
-            h = ops.decode_rmsnorm(x, L["norm1"], self.eps)
-            qkv = self._matvec(L["qkv"], h)
-            q = ops.decode_rope_append(qkv[:H], qkv[H:2 * H], qkv[2 * H:], self.cos, self.sin, position,
-                                       L["k_cache"], L["v_cache"])
-            a = ops.decode_attention(q, L["k_cache"], L["v_cache"], position, self.scale)
+            sparse = self.fuse and isinstance(L["qkv"], tuple)
+            if sparse:
+                qkv = macko_spmv.multiply_rmsnorm(L["qkv"], x, L["norm1"], self.eps)
+            else:
+                qkv = self._matvec(L["qkv"], ops.decode_rmsnorm(x, L["norm1"], self.eps))
+            if self.fuse:
+                a = ops.decode_rope_attention(qkv[:H], qkv[H:2 * H], qkv[2 * H:], self.cos, self.sin, position,
+                                              L["k_cache"], L["v_cache"], self.scale)
+            else:
+                q = ops.decode_rope_append(qkv[:H], qkv[H:2 * H], qkv[2 * H:], self.cos, self.sin, position,
+                                           L["k_cache"], L["v_cache"])
+                a = ops.decode_attention(q, L["k_cache"], L["v_cache"], position, self.scale)
             self._matvec_add(L["o"], a, x)
-            h = ops.decode_rmsnorm(x, L["norm2"], self.eps)
-            gu = self._matvec(L["gate_up"], h)
-            self._matvec_add(L["down"], ops.decode_silu_mul(gu[:I], gu[I:]), x)
+            if sparse:
+                gu = macko_spmv.multiply_rmsnorm(L["gate_up"], x, L["norm2"], self.eps)
+                macko_spmv.multiply_silu_mul_axpby(L["down"], gu[:I], gu[I:], x, 1.0, 1.0)
+            else:
+                gu = self._matvec(L["gate_up"], ops.decode_rmsnorm(x, L["norm2"], self.eps))
+                self._matvec_add(L["down"], ops.decode_silu_mul(gu[:I], gu[I:]), x)
         return torch.mv(self.lm_head, ops.decode_rmsnorm(x, self.final_norm, self.eps))
 
 
@@ -440,12 +457,15 @@ def main(argv=None):
     ap.add_argument("--module-path", action="store_true",
                     help="decode through the nn.Module forward (one framework kernel per elementary op) "
                          "instead of the lean DecodeEngine step")
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="engine path: keep rotary, the RMS norms and the SiLU gate as launches of their own")
     args = ap.parse_args(argv)
     assert torch.cuda.is_available(), "needs a GPU"
     torch.set_grad_enabled(False)
     max_len = args.prompt + args.tokens + 8
     result = {"density": args.density, "layers": args.layers, "prompt": args.prompt, "tokens": args.tokens,
-              "path": "module" if args.module_path else "engine"}
+              "path": "module" if args.module_path else "engine",
+              "fused": not (args.module_path or args.no_fuse)}
     for label, sparse in (("dense", False), ("macko", True)):
         if label == "dense" and args.skip_dense:
             continue
@@ -453,7 +473,7 @@ def main(argv=None):
                                         max_len, sparse=sparse)
         engine = None
         if not args.module_path:
-            engine = DecodeEngine(model)
+            engine = DecodeEngine(model, fuse=not args.no_fuse)
             proj_bytes = engine.weight_bytes()
             torch.cuda.empty_cache()
         resident = torch.cuda.memory_allocated()

@@ -131,13 +131,13 @@ def test_concat_compressed_equals_compressing_the_stack():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("sparse", [False, True])
-def test_engine_step_matches_module_forward(sparse):
+@pytest.mark.parametrize("sparse,fuse", [(False, False), (False, True), (True, False), (True, True)])
+def test_engine_step_matches_module_forward(sparse, fuse):
     torch.set_grad_enabled(False)
     cfg = dict(n_layers=2, dim=256, hidden=688, n_heads=4, vocab=1000, max_len=64)
     reference, _ = llm.build_model(0.5, sparse=False, **cfg)   # same seed -> same weights
     consumed, _ = llm.build_model(0.5, sparse=sparse, **cfg)
-    engine = llm.DecodeEngine(consumed)
+    engine = llm.DecodeEngine(consumed, fuse=fuse)
     prompt = torch.randint(0, 1000, (1, 10), device="cuda")
     want = reference(prompt, torch.arange(10, device="cuda"))[0].float()   # (10, vocab)
     position = torch.zeros(1, dtype=torch.long, device="cuda")
@@ -150,3 +150,25 @@ def test_engine_step_matches_module_forward(sparse):
     assert torch.equal(ids_graph, ids_eager)
     ids_module, _ = llm.greedy_decode(reference, prompt, 16, use_graph=False)
     assert (ids_module == ids_eager).float().mean() >= 0.8  # near-ties may flip an argmax
+
+
+@pytest.mark.gpu
+def test_rope_attention_equals_the_two_separate_kernels():
+    ops = torch.ops.macko_spmv
+    torch.manual_seed(11)
+    for n_heads, head_dim, max_len in ((4, 64, 40), (32, 128, 300), (3, 256, 17)):
+        half = head_dim // 2
+        ang = torch.outer(torch.arange(max_len, device="cuda").float(),
+                          1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda").float() / head_dim)))
+        cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+        kc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+        vc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+        for pos in (0, 1, max_len // 2, max_len - 1):
+            q, k, v = (torch.randn(n_heads * head_dim, device="cuda").half() for _ in range(3))
+            position = torch.tensor([pos], device="cuda")
+            kc1, vc1, kc2, vc2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+            q_rot = ops.decode_rope_append(q, k, v, cos, sin, position, kc1, vc1)
+            want = ops.decode_attention(q_rot, kc1, vc1, position, head_dim ** -0.5)
+            got = ops.decode_rope_attention(q, k, v, cos, sin, position, kc2, vc2, head_dim ** -0.5)
+            assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+            assert torch.allclose(got.float(), want.float(), rtol=1e-3, atol=1e-4)
