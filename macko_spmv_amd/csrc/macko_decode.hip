@@ -80,14 +80,18 @@ __global__ void rope_append_kernel(const uint16_t *__restrict__ q, const uint16_
     v_cache[slot + i + half] = v[in + i + half];
 }
 
-// Single-query attention over positions 0..position of one head per workgroup (256 threads):
+// Single-query attention over positions 0..position of one head per workgroup (512 threads):
 // scores, softmax, weighted sum of v.  head_dim <= 256 and a multiple of 8; max_len <= kMaxLen.
 // With ROPE the kernel first does what rope_append_kernel does for its head (q, k, v are then the
 // raw projections; the rotated q is rounded to fp16 as if it had been written out), so a decode
 // step needs one launch for both.
-constexpr int kAttnThreads = 256;
+// The kernel is latency-bound (a head's cache is a few hundred KB), so what matters is how many
+// loads are in flight: HD = head_dim as a compile-time constant lets a thread issue all loads of
+// its cache row at once (HD = 0: any head_dim, loops of runtime length), and the v pass walks four
+// positions per step.
+constexpr int kAttnThreads = 512;
 constexpr int kMaxLen = 4096;
-template <bool ROPE>
+template <bool ROPE, int HD>
 __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t *__restrict__ q,
                                                                   const uint16_t *__restrict__ k_new,
                                                                   const uint16_t *__restrict__ v_new,
@@ -95,13 +99,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
                                                                   const float *__restrict__ sin_table,
                                                                   uint16_t *k_cache, uint16_t *v_cache,
                                                                   const long long *__restrict__ position,
-                                                                  uint16_t *__restrict__ out, int head_dim, int max_len,
-                                                                  float scale)
+                                                                  uint16_t *__restrict__ out, int head_dim_arg,
+                                                                  int max_len, float scale)
 {
     __shared__ float scores[kMaxLen];
-    __shared__ float qs[256];
-    __shared__ float partial[kAttnThreads * 8];  // groups x head_dim <= 2048
+    __shared__ __attribute__((aligned(16))) float qs[256];
+    __shared__ float partial[kAttnThreads * 8];  // groups x head_dim
     __shared__ float scratch[17];
+    const int head_dim = HD ? HD : head_dim_arg;
     const int head = blockIdx.x, tid = threadIdx.x;
     long long pos = position[0];
     pos = pos < 0 ? 0 : (pos >= max_len ? max_len - 1 : pos);
@@ -129,17 +134,26 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
     __syncthreads();
     const uint16_t *kh = k_cache + (size_t)head * max_len * head_dim;
     const uint16_t *vh = v_cache + (size_t)head * max_len * head_dim;
+    auto dot8 = [&](const u32x4 kv, int j, float acc) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            acc += h2f((uint16_t)(kv[e] & 0xffffu)) * qs[8 * j + 2 * e];
+            acc += h2f((uint16_t)(kv[e] >> 16)) * qs[8 * j + 2 * e + 1];
+        }
+        return acc;
+    };
     float local_max = -3.0e38f;
     for (int p = tid; p < len; p += kAttnThreads) {
         const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)p * head_dim);
         float acc = 0.f;
-        for (int j = 0; j < head_dim / 8; ++j) {
-            const u32x4 kv = row[j];
+        if (HD > 0) {
+            u32x4 kv[HD > 0 ? HD / 8 : 1];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc += h2f((uint16_t)(kv[e] & 0xffffu)) * qs[8 * j + 2 * e];
-                acc += h2f((uint16_t)(kv[e] >> 16)) * qs[8 * j + 2 * e + 1];
-            }
+            for (int j = 0; j < HD / 8; ++j) kv[j] = row[j];
+#pragma unroll
+            for (int j = 0; j < HD / 8; ++j) acc = dot8(kv[j], j, acc);
+        } else {
+            for (int j = 0; j < head_dim / 8; ++j) acc = dot8(row[j], j, acc);
         }
         scores[p] = acc;
         local_max = fmaxf(local_max, acc);
@@ -159,13 +173,23 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
     const int g = tid / lanes_per_row, j = tid - g * lanes_per_row;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (g < groups) {
-        for (int p = g; p < len; p += groups) {
-            const float wgt = scores[p];
-            const u32x4 vv = reinterpret_cast<const u32x4 *>(vh + (size_t)p * head_dim)[j];
+        for (int p = g; p < len; p += 4 * groups) {
+            u32x4 vv[4];
+            float wgt[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc[2 * e] += wgt * h2f((uint16_t)(vv[e] & 0xffffu));
-                acc[2 * e + 1] += wgt * h2f((uint16_t)(vv[e] >> 16));
+            for (int u = 0; u < 4; ++u) {
+                const int pu = p + u * groups;
+                const bool ok = pu < len;
+                vv[u] = ok ? reinterpret_cast<const u32x4 *>(vh + (size_t)pu * head_dim)[j] : u32x4{0, 0, 0, 0};
+                wgt[u] = ok ? scores[pu] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[2 * e] += wgt[u] * h2f((uint16_t)(vv[u][e] & 0xffffu));
+                    acc[2 * e + 1] += wgt[u] * h2f((uint16_t)(vv[u][e] >> 16));
+                }
             }
         }
 #pragma unroll
@@ -177,6 +201,25 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
         for (int gg = 0; gg < groups; ++gg) total += partial[gg * head_dim + tid];
         out[(size_t)head * head_dim + tid] = f2h(total * inv);
     }
+}
+
+template <bool ROPE>
+void launch_attention(const void *q, const void *k, const void *v, const float *cos_table, const float *sin_table,
+                      void *k_cache, void *v_cache, const int64_t *position, void *out, int n_heads, int head_dim,
+                      int max_len, float scale, hipStream_t stream)
+{
+#define MACKO_ATTN(HD_)                                                                                         \
+    hipLaunchKernelGGL((attention_kernel<ROPE, HD_>), dim3(n_heads), dim3(kAttnThreads), 0, stream,             \
+                       (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, cos_table, sin_table,      \
+                       (uint16_t *)k_cache, (uint16_t *)v_cache, (const long long *)position, (uint16_t *)out,   \
+                       head_dim, max_len, scale)
+    if (head_dim == 128)
+        MACKO_ATTN(128);
+    else if (head_dim == 64)
+        MACKO_ATTN(64);
+    else
+        MACKO_ATTN(0);
+#undef MACKO_ATTN
 }
 
 // out[i] = silu(gate[i]) * up[i]
@@ -229,11 +272,9 @@ extern "C" int macko_decode_attention_f16(const void *q, const void *k_cache, co
         return MACKO_E_INVALID_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(k_cache) & 15) || (reinterpret_cast<uintptr_t>(v_cache) & 15))
         return MACKO_E_INVALID_ARGUMENT;
-    hipLaunchKernelGGL(attention_kernel<false>, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
-                       (const uint16_t *)q, (const uint16_t *)nullptr, (const uint16_t *)nullptr,
-                       (const float *)nullptr, (const float *)nullptr, (uint16_t *)const_cast<void *>(k_cache),
-                       (uint16_t *)const_cast<void *>(v_cache), (const long long *)position, (uint16_t *)out,
-                       head_dim, max_len, scale);
+    launch_attention<false>(q, nullptr, nullptr, nullptr, nullptr, const_cast<void *>(k_cache),
+                            const_cast<void *>(v_cache), position, out, n_heads, head_dim, max_len, scale,
+                            as_stream(stream));
     return (int)hipGetLastError();
 }
 
@@ -249,10 +290,8 @@ extern "C" int macko_decode_rope_attention_f16(const void *q, const void *k, con
         return MACKO_E_INVALID_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(k_cache) & 15) || (reinterpret_cast<uintptr_t>(v_cache) & 15))
         return MACKO_E_INVALID_ARGUMENT;
-    hipLaunchKernelGGL(attention_kernel<true>, dim3(n_heads), dim3(kAttnThreads), 0, as_stream(stream),
-                       (const uint16_t *)q, (const uint16_t *)k, (const uint16_t *)v, cos_table, sin_table,
-                       (uint16_t *)k_cache, (uint16_t *)v_cache, (const long long *)position, (uint16_t *)out,
-                       head_dim, max_len, scale);
+    launch_attention<true>(q, k, v, cos_table, sin_table, k_cache, v_cache, position, out, n_heads, head_dim,
+                           max_len, scale, as_stream(stream));
     return (int)hipGetLastError();
 }
 
