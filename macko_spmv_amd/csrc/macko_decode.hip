@@ -84,13 +84,15 @@ __global__ void rope_append_kernel(const uint16_t *__restrict__ q, const uint16_
 // scores, softmax, weighted sum of v.  head_dim <= 256 and a multiple of 8; max_len <= kMaxLen.
 // With ROPE the kernel first does what rope_append_kernel does for its head (q, k, v are then the
 // raw projections; the rotated q is rounded to fp16 as if it had been written out), so a decode
-// step needs one launch for both.
-// The kernel is latency-bound (a head's cache is a few hundred KB), so what matters is how many
-// loads are in flight: HD = head_dim as a compile-time constant lets a thread issue all loads of
-// its cache row at once (HD = 0: any head_dim, loops of runtime length), and the v pass walks four
-// positions per step.
+// step needs one launch for both.  The row it appends is used from LDS, not read back.
+// The kernel is latency-bound (a head's cache is a few hundred KB), so what matters is how few
+// dependent memory round trips there are: HD = head_dim as a compile-time constant lets a thread
+// issue all loads of its k row at once (HD = 0: any head_dim, loops of runtime length), and the k
+// row of a thread's first position and the v pieces of its first kVPre positions are requested
+// before anything else is computed, together with q, k, v of the new token.
 constexpr int kAttnThreads = 512;
 constexpr int kMaxLen = 4096;
+constexpr int kVPre = 8;
 template <bool ROPE, int HD>
 __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t *__restrict__ q,
                                                                   const uint16_t *__restrict__ k_new,
@@ -104,6 +106,8 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
 {
     __shared__ float scores[kMaxLen];
     __shared__ __attribute__((aligned(16))) float qs[256];
+    __shared__ __attribute__((aligned(16))) uint16_t ks[256];  // the appended row (ROPE only)
+    __shared__ __attribute__((aligned(16))) uint16_t vs[256];
     __shared__ float partial[kAttnThreads * 8];  // groups x head_dim
     __shared__ float scratch[17];
     const int head_dim = HD ? HD : head_dim_arg;
@@ -111,6 +115,31 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
     long long pos = position[0];
     pos = pos < 0 ? 0 : (pos >= max_len ? max_len - 1 : pos);
     const int len = (int)pos + 1;
+    const int own = ROPE ? (int)pos : -1;  // the row this launch appends
+    const uint16_t *kh = k_cache + (size_t)head * max_len * head_dim;
+    const uint16_t *vh = v_cache + (size_t)head * max_len * head_dim;
+    const int lanes_per_row = head_dim >> 3;
+    const int groups = kAttnThreads / lanes_per_row;
+    const int g = tid / lanes_per_row, j = tid - g * lanes_per_row;
+
+    // ---- cache loads that depend on nothing computed here -------------------------------------------
+    constexpr int NV = HD > 0 ? HD / 8 : 1;
+    u32x4 kpre[NV];
+    if (HD > 0) {
+        const bool fetch = tid < len && tid != own;
+        const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)tid * head_dim);
+#pragma unroll
+        for (int jj = 0; jj < NV; ++jj) kpre[jj] = fetch ? row[jj] : u32x4{0, 0, 0, 0};
+    }
+    u32x4 vpre[kVPre];
+#pragma unroll
+    for (int u = 0; u < kVPre; ++u) {
+        const int pu = g + u * groups;
+        const bool fetch = g < groups && pu < len && pu != own;
+        vpre[u] = fetch ? reinterpret_cast<const u32x4 *>(vh + (size_t)pu * head_dim)[j] : u32x4{0, 0, 0, 0};
+    }
+
+    // ---- q (rotated with ROPE), and the new cache row -------------------------------------------------
     if (ROPE) {
         const int half = head_dim >> 1;
         if (tid < half) {
@@ -122,38 +151,47 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
             qs[i] = h2f(f2h(q0 * c - q1 * s)) * scale;
             qs[i + half] = h2f(f2h(q1 * c + q0 * s)) * scale;
             const float k0 = h2f(k_new[in + i]), k1 = h2f(k_new[in + i + half]);
-            k_cache[slot + i] = f2h(k0 * c - k1 * s);
-            k_cache[slot + i + half] = f2h(k1 * c + k0 * s);
-            v_cache[slot + i] = v_new[in + i];
-            v_cache[slot + i + half] = v_new[in + i + half];
+            const uint16_t r0 = f2h(k0 * c - k1 * s), r1 = f2h(k1 * c + k0 * s);
+            const uint16_t v0 = v_new[in + i], v1 = v_new[in + i + half];
+            ks[i] = r0;
+            ks[i + half] = r1;
+            vs[i] = v0;
+            vs[i + half] = v1;
+            k_cache[slot + i] = r0;
+            k_cache[slot + i + half] = r1;
+            v_cache[slot + i] = v0;
+            v_cache[slot + i + half] = v1;
         }
-        __threadfence();  // the new cache row is read back below by other threads of this workgroup
     } else if (tid < head_dim) {
         qs[tid] = h2f(q[(size_t)head * head_dim + tid]) * scale;
     }
     __syncthreads();
-    const uint16_t *kh = k_cache + (size_t)head * max_len * head_dim;
-    const uint16_t *vh = v_cache + (size_t)head * max_len * head_dim;
-    auto dot8 = [&](const u32x4 kv, int j, float acc) {
+
+    // ---- scores -----------------------------------------------------------------------------------------
+    auto dot8 = [&](const u32x4 kv, int jj, float acc) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            acc += h2f((uint16_t)(kv[e] & 0xffffu)) * qs[8 * j + 2 * e];
-            acc += h2f((uint16_t)(kv[e] >> 16)) * qs[8 * j + 2 * e + 1];
+            acc += h2f((uint16_t)(kv[e] & 0xffffu)) * qs[8 * jj + 2 * e];
+            acc += h2f((uint16_t)(kv[e] >> 16)) * qs[8 * jj + 2 * e + 1];
         }
         return acc;
     };
     float local_max = -3.0e38f;
     for (int p = tid; p < len; p += kAttnThreads) {
-        const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)p * head_dim);
         float acc = 0.f;
-        if (HD > 0) {
-            u32x4 kv[HD > 0 ? HD / 8 : 1];
+        if (p == own) {
+            for (int jj = 0; jj < lanes_per_row; ++jj) acc = dot8(reinterpret_cast<const u32x4 *>(ks)[jj], jj, acc);
+        } else if (HD > 0) {
+            if (p != tid) {  // beyond the row requested up front
+                const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)p * head_dim);
 #pragma unroll
-            for (int j = 0; j < HD / 8; ++j) kv[j] = row[j];
+                for (int jj = 0; jj < NV; ++jj) kpre[jj] = row[jj];
+            }
 #pragma unroll
-            for (int j = 0; j < HD / 8; ++j) acc = dot8(kv[j], j, acc);
+            for (int jj = 0; jj < NV; ++jj) acc = dot8(kpre[jj], jj, acc);
         } else {
-            for (int j = 0; j < head_dim / 8; ++j) acc = dot8(row[j], j, acc);
+            const u32x4 *row = reinterpret_cast<const u32x4 *>(kh + (size_t)p * head_dim);
+            for (int jj = 0; jj < lanes_per_row; ++jj) acc = dot8(row[jj], jj, acc);
         }
         scores[p] = acc;
         local_max = fmaxf(local_max, acc);
@@ -166,31 +204,37 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
         local_sum += e;
     }
     const float inv = 1.0f / block_sum(local_sum, scratch);  // also orders the scores[] writes
-    // Weighted sum of v: a thread owns 8 consecutive dims (one 16-byte load per position) of the
-    // positions p = g, g + groups, ...; the groups' partial sums meet in LDS.
-    const int lanes_per_row = head_dim >> 3;
-    const int groups = kAttnThreads / lanes_per_row;
-    const int g = tid / lanes_per_row, j = tid - g * lanes_per_row;
+
+    // ---- weighted sum of v: a thread owns 8 consecutive dims (one 16-byte piece per position) of the
+    //      positions p = g, g + groups, ...; the groups' partial sums meet in LDS --------------------------
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    auto add_row = [&](const u32x4 vv, float wgt) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            acc[2 * e] += wgt * h2f((uint16_t)(vv[e] & 0xffffu));
+            acc[2 * e + 1] += wgt * h2f((uint16_t)(vv[e] >> 16));
+        }
+    };
     if (g < groups) {
-        for (int p = g; p < len; p += 4 * groups) {
+#pragma unroll
+        for (int u = 0; u < kVPre; ++u) {
+            const int pu = g + u * groups;
+            if (pu < len) add_row(pu == own ? reinterpret_cast<const u32x4 *>(vs)[j] : vpre[u], scores[pu]);
+        }
+        for (int p = g + kVPre * groups; p < len; p += 4 * groups) {
             u32x4 vv[4];
             float wgt[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int pu = p + u * groups;
                 const bool ok = pu < len;
-                vv[u] = ok ? reinterpret_cast<const u32x4 *>(vh + (size_t)pu * head_dim)[j] : u32x4{0, 0, 0, 0};
+                vv[u] = !ok ? u32x4{0, 0, 0, 0}
+                            : (pu == own ? reinterpret_cast<const u32x4 *>(vs)[j]
+                                         : reinterpret_cast<const u32x4 *>(vh + (size_t)pu * head_dim)[j]);
                 wgt[u] = ok ? scores[pu] : 0.f;
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc[2 * e] += wgt[u] * h2f((uint16_t)(vv[u][e] & 0xffffu));
-                    acc[2 * e + 1] += wgt[u] * h2f((uint16_t)(vv[u][e] >> 16));
-                }
-            }
+            for (int u = 0; u < 4; ++u) add_row(vv[u], wgt[u]);
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) partial[g * head_dim + 8 * j + e] = acc[e];
