@@ -57,7 +57,9 @@ extern "C" int macko_calibration_copy(const void *src, void *dst, int64_t bytes,
 }
 
 // Pure streaming read in the SpMV's own access shape: 256 x 1024 threads, every wave walks one
-// contiguous 1/4096 of the buffer with two 16-byte loads per lane in flight.  What it takes is the
+// contiguous 1/4096 of the buffer with four non-temporal 16-byte loads per lane in flight (the
+// fastest of the read patterns tried: span per wave or per workgroup, grid stride, 2 to 8 loads in
+// flight, with and without the hint).  What it takes is the
 // time any one-launch kernel needs just to pull `bytes` out of HBM: the yardstick the benchmark
 // prints next to the SpMV's time.
 __global__ void __launch_bounds__(1024) calibration_read_kernel(const macko::u32x4 *__restrict__ src, size_t n_vec,
@@ -68,12 +70,15 @@ __global__ void __launch_bounds__(1024) calibration_read_kernel(const macko::u32
     const size_t begin = n_vec * w / n_waves, end = n_vec * (w + 1) / n_waves;
     macko::u32 acc = 0;
     size_t i = begin + lane;
-    for (; i + 64 < end; i += 128) {
-        const macko::u32x4 a = src[i], b = src[i + 64];
-        acc += a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
+    for (; i + 192 < end; i += 256) {
+        macko::u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = __builtin_nontemporal_load(&src[i + 64 * k]);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc += v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
     }
     for (; i < end; i += 64) {
-        const macko::u32x4 a = src[i];
+        const macko::u32x4 a = __builtin_nontemporal_load(&src[i]);
         acc += a.x ^ a.y ^ a.z ^ a.w;
     }
     if (acc == 0x9e3779b9u) *sink = acc;  // keeps the loads alive; practically never true

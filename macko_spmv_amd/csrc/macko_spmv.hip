@@ -298,9 +298,13 @@ __device__ __forceinline__ void xpiece_to_lds(u32 lds_byte_address)
     if (J == 1) asm volatile("s_waitcnt vmcnt(%1)\n\tds_write_b128 %0, v[84:87]" ::"v"(lds_byte_address), "n"(N) : "memory");
 }
 
-// ring slot J of a D-deep ring: issue both loads / wait and copy out
-#define MACKO_RING_ISSUE(VREGS, DREG, CLOBBERS)                                                            \
-    asm volatile("buffer_load_dwordx4 " VREGS ", %0, %2, 0 offen\n\tbuffer_load_dword " DREG ", %1, %3, 0 offen" \
+// ring slot J of a D-deep ring: issue both loads / wait and copy out.  HINT is "" or " nt": the
+// matrix is read once per product, and a streaming read of that kind measures 11% faster with the
+// non-temporal hint at a few hundred MB.  Tiles a wave shares with a neighbour (its first and last)
+// go without it, so the second reader still finds them in L2.
+#define MACKO_RING_ISSUE(VREGS, DREG, HINT, CLOBBERS)                                                       \
+    asm volatile("buffer_load_dwordx4 " VREGS ", %0, %2, 0 offen" HINT "\n\tbuffer_load_dword " DREG         \
+                 ", %1, %3, 0 offen" HINT                                                                   \
                  ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
                  : "memory", CLOBBERS)
 #define MACKO_RING_TAKE(A, B, C, E, DREG)                                                                      \
@@ -308,32 +312,41 @@ __device__ __forceinline__ void xpiece_to_lds(u32 lds_byte_address)
                  "\n\tv_mov_b32 %3, " E "\n\tv_mov_b32 %4, " DREG                                               \
                  : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w), "=v"(d) : "n"(N) : "memory")
 
-#define MACKO_RING_ISSUE_I8(VREGS, DREG, CLOBBERS)                                                         \
-    asm volatile("buffer_load_dwordx2 " VREGS ", %0, %2, 0 offen\n\tbuffer_load_dword " DREG ", %1, %3, 0 offen" \
+#define MACKO_RING_ISSUE_I8(VREGS, DREG, HINT, CLOBBERS)                                                    \
+    asm volatile("buffer_load_dwordx2 " VREGS ", %0, %2, 0 offen" HINT "\n\tbuffer_load_dword " DREG         \
+                 ", %1, %3, 0 offen" HINT                                                                   \
                  ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
                  : "memory", CLOBBERS)
+// `stream` is wave-uniform
+#define MACKO_RING_ISSUE_EITHER(MACRO, VREGS, DREG)                \
+    do {                                                           \
+        if (stream)                                                \
+            MACRO(VREGS, DREG, " nt", MACKO_FIXED_CLOBBERS_4);     \
+        else                                                       \
+            MACRO(VREGS, DREG, "", MACKO_FIXED_CLOBBERS_4);        \
+    } while (0)
 
 // VB = bytes per stored value: 2 (fp16, 16 bytes per lane and tile) or 1 (int8, 8 bytes per lane
 // and tile, which land in the first two registers of the slot).
 template <int D, int J, int VB>
 __device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
-                                           const u32x4 &buf_deltas)
+                                           const u32x4 &buf_deltas, bool stream)
 {
     static_assert(D == 1 || D == 2 || D == 4, "ring depth");
     static_assert(VB == 2 || (VB == 1 && D <= 2), "the int8 ring exists at depth 1 and 2 only");
     if (VB == 1) {
-        if (D == 1 && J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v92", MACKO_FIXED_CLOBBERS_4);
-        if (D == 2 && J == 0) MACKO_RING_ISSUE_I8("v[88:89]", "v96", MACKO_FIXED_CLOBBERS_4);
-        if (D == 2 && J == 1) MACKO_RING_ISSUE_I8("v[92:93]", "v97", MACKO_FIXED_CLOBBERS_4);
+        if (D == 1 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[88:89]", "v92");
+        if (D == 2 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[88:89]", "v96");
+        if (D == 2 && J == 1) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[92:93]", "v97");
         return;
     }
-    if (D == 1 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v92", MACKO_FIXED_CLOBBERS_4);
-    if (D == 2 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v96", MACKO_FIXED_CLOBBERS_4);
-    if (D == 2 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v97", MACKO_FIXED_CLOBBERS_4);
-    if (D == 4 && J == 0) MACKO_RING_ISSUE("v[88:91]", "v104", MACKO_FIXED_CLOBBERS_4);
-    if (D == 4 && J == 1) MACKO_RING_ISSUE("v[92:95]", "v105", MACKO_FIXED_CLOBBERS_4);
-    if (D == 4 && J == 2) MACKO_RING_ISSUE("v[96:99]", "v106", MACKO_FIXED_CLOBBERS_4);
-    if (D == 4 && J == 3) MACKO_RING_ISSUE("v[100:103]", "v107", MACKO_FIXED_CLOBBERS_4);
+    if (D == 1 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[88:91]", "v92");
+    if (D == 2 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[88:91]", "v96");
+    if (D == 2 && J == 1) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[92:95]", "v97");
+    if (D == 4 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[88:91]", "v104");
+    if (D == 4 && J == 1) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[92:95]", "v105");
+    if (D == 4 && J == 2) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[96:99]", "v106");
+    if (D == 4 && J == 3) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[100:103]", "v107");
 }
 
 template <int D, int J, int N>
@@ -410,10 +423,10 @@ spmv_stream_kernel(const SpmvArgs a)
         xpiece_issue<0>((u32)tid * 16, buf_x);
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
-    auto issue_slot = [&](auto slot, u32 tile, bool fetch) {
+    auto issue_slot = [&](auto slot, u32 tile, bool fetch, bool stream) {
         constexpr int J = decltype(slot)::value;
         ring_issue<D, J, VB>(lane_values + (fetch ? tile * (u32)(kTile * VB) : kNoTileValues),
-                         lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas);
+                         lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas, stream);
     };
     // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
     //         x, goes to LDS through ordinary loads (rare: more than 16384 columns, or an x that is
@@ -645,7 +658,8 @@ spmv_stream_kernel(const SpmvArgs a)
         last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
         static_for<D>([&](auto slot) {
             constexpr int J = decltype(slot)::value;
-            issue_slot(slot, first_tile + J, first_tile + J < last_tile);
+            // my first and last tile may be shared with a neighbouring wave: no streaming hint there
+            issue_slot(slot, first_tile + J, first_tile + J < last_tile, J > 0 && first_tile + J + 1 < last_tile);
         });
     }
 
@@ -818,7 +832,7 @@ spmv_stream_kernel(const SpmvArgs a)
             u32x4 vj;
             u32 dj;
             ring_take<D, J, kTileLoads - 2>(vj, dj);
-            issue_slot(slot, tile + D, tile + D < last_tile);  // refill at once: the copy is out
+            issue_slot(slot, tile + D, tile + D < last_tile, tile + D + 1 < last_tile);  // refill at once: the copy is out
             const int tb = (int)(tile << kTileShift);
             const int tile_end = tb + kTile;
             if (e0 <= tb && e1 >= tile_end) {  // the common case for rows longer than a tile
@@ -910,12 +924,10 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     if (grid > (long long)info.compute_units * wg_per_cu) grid = (long long)info.compute_units * wg_per_cu;
     if (grid < 1) grid = 1;
     // Ring depth: one tile in flight behind the one being processed is enough, and cheapest to
-    // start, when a wave owns a single row or only a few tiles; waves that walk many tiles over
-    // several rows do slightly better with two (measured on the Llama shapes; deeper is slower).
+    // start, when a wave walks only a few tiles; from about four tiles per wave on, two do better
+    // (measured on the Llama shapes and larger ones, fp16 and int8; deeper is slower).
     const long long n_waves = grid * waves;
-    // The int8 variant, whose tiles are 40% smaller, takes two whenever the walk is long (measured).
-    const bool long_walk = n_tiles >= 6 * n_waves;
-    const int depth = t.depth ? t.depth : (long_walk && (VB == 1 || (long long)a.rows > n_waves) ? 2 : 1);
+    const int depth = t.depth ? t.depth : (n_tiles >= 4 * n_waves ? 2 : 1);
 
     const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack) + (XF == 1 ? 64 : 0);
     if (XF != 0) {  // fused staging: x must fit in LDS (checked by the caller too)
