@@ -36,7 +36,7 @@ LARGE_DENSITIES = [0.1, 0.3, 0.5]
 # default workload: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, each scaled by what the
 # same counter reports for calibration_copy_kernel on 256 MiB (factors 0.5000 and 1.0000).  Source:
 # profiles/spmv_stream_kernel_llama_shapes_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 42.81e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 40.80e6}
 
 WORKLOADS = {
     "llama": "configs[1]: Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as fp16 SpMV, per-row "
@@ -452,7 +452,7 @@ def main():
         t_r = sum(p["stream_read_us"] for p in per_case)
         yardstick = {
             "what": "calibration_read_kernel: one launch that only reads the same number of bytes (256x1024 "
-                    "threads, contiguous span per wave), timed like the per-case SpMV figures",
+                    "threads, contiguous span per wave, four non-temporal 16-byte loads per lane in flight), timed like the per-case SpMV figures",
             "us_per_launch": round(t_r / len(per_case), 3),
             "gbps": round(step_bytes / t_r / 1e3, 1),
             "spmv_time_over_read_time": round(t_m / t_r, 3),
