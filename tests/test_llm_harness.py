@@ -82,7 +82,7 @@ def test_glue_kernels_match_torch_fp32():
         g, u = torch.randn(n, device="cuda").half(), torch.randn(n, device="cuda").half()
         want = torch.nn.functional.silu(g.float()) * u.float()
         assert torch.allclose(ops.decode_silu_mul(g, u).float(), want, rtol=2e-3, atol=2e-3)
-    for n_heads, head_dim, max_len, pos in ((4, 64, 48, 0), (32, 128, 400, 37), (2, 16, 300, 299), (3, 96, 700, 511)):
+    for n_heads, head_dim, max_len, pos in ((4, 64, 48, 0), (32, 128, 400, 37), (2, 16, 300, 299), (3, 96, 700, 511), (2, 128, 2048, 2047), (2, 64, 1500, 1100)):
         H = n_heads * head_dim
         q, k, v = (torch.randn(H, device="cuda").half() for _ in range(3))
         inv = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda").float() / head_dim))
@@ -156,7 +156,7 @@ def test_engine_step_matches_module_forward(sparse, fuse):
 def test_rope_attention_equals_the_two_separate_kernels():
     ops = torch.ops.macko_spmv
     torch.manual_seed(11)
-    for n_heads, head_dim, max_len in ((4, 64, 40), (32, 128, 300), (3, 256, 17)):
+    for n_heads, head_dim, max_len in ((4, 64, 40), (32, 128, 300), (3, 256, 17), (2, 128, 1300), (2, 80, 700)):
         half = head_dim // 2
         ang = torch.outer(torch.arange(max_len, device="cuda").float(),
                           1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda").float() / head_dim)))
