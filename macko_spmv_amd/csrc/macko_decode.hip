@@ -15,11 +15,12 @@ __device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_c
 __device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 
 // Sum over the workgroup (blockDim.x a multiple of 64, at most 1024); every thread gets the total.
-__device__ __forceinline__ float block_sum(float v, float *scratch /* [17] */)
+// `scratch` is 16 floats that no other reduction of the same kernel uses (so no barrier is needed
+// in front of the write).
+__device__ __forceinline__ float block_sum(float v, float *scratch)
 {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
     const float w = wave_sum(v);
-    __syncthreads();  // scratch may still be read from an earlier call
     if (lane == 0) scratch[wave] = w;
     __syncthreads();
     float total = 0.f;
@@ -33,7 +34,6 @@ __device__ __forceinline__ float block_max(float v, float *scratch)
     float m = v;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    __syncthreads();
     if (lane == 0) scratch[wave] = m;
     __syncthreads();
     float total = scratch[0];
@@ -45,7 +45,7 @@ __device__ __forceinline__ float block_max(float v, float *scratch)
 __global__ void __launch_bounds__(1024) rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
                                                        uint16_t *__restrict__ y, int n, float eps)
 {
-    __shared__ float scratch[17];
+    __shared__ float scratch[16];
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const float v = h2f(x[i]);
@@ -109,7 +109,7 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
     __shared__ __attribute__((aligned(16))) uint16_t ks[256];  // the appended row (ROPE only)
     __shared__ __attribute__((aligned(16))) uint16_t vs[256];
     __shared__ float partial[kAttnThreads * 8];  // groups x head_dim
-    __shared__ float scratch[17];
+    __shared__ float max_scratch[16], sum_scratch[16];
     const int head_dim = HD ? HD : head_dim_arg;
     const int head = blockIdx.x, tid = threadIdx.x;
     long long pos = position[0];
@@ -196,14 +196,14 @@ __global__ void __launch_bounds__(kAttnThreads) attention_kernel(const uint16_t 
         scores[p] = acc;
         local_max = fmaxf(local_max, acc);
     }
-    const float m = block_max(local_max, scratch);
+    const float m = block_max(local_max, max_scratch);
     float local_sum = 0.f;
     for (int p = tid; p < len; p += kAttnThreads) {
         const float e = __expf(scores[p] - m);
         scores[p] = e;
         local_sum += e;
     }
-    const float inv = 1.0f / block_sum(local_sum, scratch);  // also orders the scores[] writes
+    const float inv = 1.0f / block_sum(local_sum, sum_scratch);  // also orders the scores[] writes
 
     // ---- weighted sum of v: a thread owns 8 consecutive dims (one 16-byte piece per position) of the
     //      positions p = g, g + groups, ...; the groups' partial sums meet in LDS --------------------------
