@@ -172,3 +172,31 @@ def test_rope_attention_equals_the_two_separate_kernels():
             got = ops.decode_rope_attention(q, k, v, cos, sin, position, kc2, vc2, head_dim ** -0.5)
             assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
             assert torch.allclose(got.float(), want.float(), rtol=1e-3, atol=1e-4)
+
+
+def test_concat_compressed_against_the_oracle_on_the_host():
+    # pure tensor logic, so it runs without a GPU: parts compressed by the CPU oracle, stacked, and
+    # compared with the oracle's compression of the stacked dense matrix (odd entry counts make the
+    # nibble stream of the following part start on a high nibble; one part is entirely empty)
+    import numpy as np
+
+    from oracle import macko_oracle as mo
+    from tests import helpers
+
+    rng = np.random.default_rng(17)
+    mats = [helpers.random_sparse(rng, rows, 203, dens) for rows, dens in ((5, 0.3), (9, 0.05), (4, 0.0), (17, 0.6), (1, 1.0))]
+    mats[0][2] = 0
+
+    def as_tuple(dense):
+        values, deltas, row_ptr, _ = mo.compress(dense)
+        return (torch.from_numpy(values.view(np.float16).copy()), torch.from_numpy(deltas.copy()),
+                torch.from_numpy(row_ptr.copy()), dense.shape[0], dense.shape[1])
+
+    assert any(int(as_tuple(m)[2][-1]) % 2 == 1 for m in mats[:-1]), "no part with an odd entry count"
+    got = llm.concat_compressed([as_tuple(m) for m in mats])
+    want = as_tuple(np.concatenate(mats, axis=0))
+    assert got[3] == want[3] and got[4] == want[4]
+    for a, b in zip(got[:3], want[:3]):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert torch.equal(a.view(torch.int16) if a.dtype == torch.float16 else a,
+                           b.view(torch.int16) if b.dtype == torch.float16 else b)
