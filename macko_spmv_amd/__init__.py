@@ -26,9 +26,9 @@ LIB_NAME = "macko_spmv"
 
 def _load_native():
     hip_path, torch_path = _build.lib_paths()
-    if not (os.path.exists(hip_path) and os.path.exists(torch_path)):
-        # first use: compile in place, like the upstream package's JIT step at import
-        # (src/macko_spmv/__init__.py:14-102)
+    if not _build.is_current():
+        # first use, or the sources have changed since the libraries were built: compile in place,
+        # like the upstream package's JIT step at import (src/macko_spmv/__init__.py:14-102)
         _build.build_all()
     try:
         hip = ctypes.CDLL(hip_path, mode=ctypes.RTLD_GLOBAL)

@@ -25,7 +25,7 @@ HIP_LIB = "libmacko_hip.so"
 TORCH_LIB = "libmacko_torch.so"
 ARCH = "gfx950"
 
-HIP_SOURCES = ["macko_spmv.hip", "macko_compress.hip", "macko_runtime.hip", "macko_decode.hip"]
+HIP_SOURCES = ["macko_spmv.hip", "macko_spmv_split.hip", "macko_compress.hip", "macko_runtime.hip", "macko_decode.hip"]
 TORCH_SOURCES = ["macko_torch.cpp"]
 
 
@@ -67,24 +67,29 @@ _DEVICE_FLAGS = [
     f"-I{_INCLUDE}", f"-I{_CSRC}",
 ]
 
-# The SpMV kernel keeps its in-flight loads in fixed VGPRs from this one up (kCompilerVgprs in
-# macko_spmv.hip); compiler-generated code must stay below it.
-FIXED_VGPR_BASE = 78
+# The SpMV kernels keep their in-flight loads in fixed VGPRs from a certain register up
+# (kCompilerVgprs in their source files); compiler-generated code must stay below it.
+# source file -> (kernel name, first fixed VGPR, first register of every ring slot)
+TRACKED_KERNELS = {
+    "macko_spmv.hip": ("spmv_stream_kernel", 78, (88, 92, 96, 100)),
+    "macko_spmv_split.hip": ("spmv_split_kernel", 84, (94, 98)),
+}
 
 
-def check_stream_kernel_assembly(text):
-    """`text`: lines of the assembly of macko_spmv.hip.  Checks two things the hand-tracked loads of
-    every spmv_stream_kernel rely on: outside the hand-written asm blocks no instruction touches a
-    VGPR >= FIXED_VGPR_BASE, and the compiler has put no vmcnt wait of its own right in front of a
-    ring take (it does when one of its own loads may still be outstanding at the loop's back edge;
-    such a wait also waits for the ring loads in flight and serialises the stream).  Returns the
-    number of kernels checked; raises RuntimeError on a violation."""
+def check_stream_kernel_assembly(text, kernel_name="spmv_stream_kernel", fixed_base=78, slot_registers=(88, 92, 96, 100)):
+    """`text`: lines of the assembly of one of the SpMV source files.  Checks two things the
+    hand-tracked loads of every instantiation of `kernel_name` rely on: outside the hand-written asm
+    blocks no instruction touches a VGPR >= fixed_base, and the compiler has put no vmcnt wait of its
+    own right in front of a ring take (it does when one of its own loads may still be outstanding at
+    the loop's back edge; such a wait also waits for the ring loads in flight and serialises the
+    stream).  Returns the number of kernels checked; raises RuntimeError on a violation."""
     kernel = None
     in_asm = False
     checked = 0
     recent_wait = None  # (line number, text) of the last compiler-generated vmcnt wait
+    take = re.compile(r"v_mov_b32 \S+ v(%s)\b" % "|".join(str(r) for r in slot_registers))
     for number, line in enumerate(text):
-        m = re.match(r"^(_Z\S*spmv_stream_kernel\S*):", line)
+        m = re.match(r"^(_Z\S*%s\S*):" % kernel_name, line)
         if m:
             kernel, in_asm, recent_wait = m.group(1), False, None
             checked += 1
@@ -98,8 +103,8 @@ def check_stream_kernel_assembly(text):
         elif "#ASMEND" in line:
             in_asm = False
         elif in_asm:
-            # a ring take copies out of v88.. after its own wait
-            if recent_wait and number - recent_wait[0] <= 16 and re.search(r"v_mov_b32 \S+ v(88|92|96|100)\b", line):
+            # a ring take copies out of its slot's registers after its own wait
+            if recent_wait and number - recent_wait[0] <= 16 and take.search(line):
                 raise RuntimeError(f"compiler-generated '{recent_wait[1]}' in front of a ring take in {kernel} "
                                    f"(assembly line {recent_wait[0] + 1})")
         else:
@@ -110,33 +115,75 @@ def check_stream_kernel_assembly(text):
                 recent_wait = (number, code.strip())
             regs = [int(b) for _, b in re.findall(r"\bv\[(\d+):(\d+)\]", code)]
             regs += [int(a) for a in re.findall(r"\bv(\d+)\b", code)]
-            if regs and max(regs) >= FIXED_VGPR_BASE:
+            if regs and max(regs) >= fixed_base:
                 raise RuntimeError(f"compiler-generated code touches a fixed VGPR in {kernel}: {line.strip()}")
     if checked == 0:
-        raise RuntimeError("no spmv_stream_kernel found in the assembly; the register check is stale")
+        raise RuntimeError(f"no {kernel_name} found in the assembly; the register check is stale")
     return checked
 
 
 def verify_fixed_registers(verbose=False):
-    """Compile macko_spmv.hip to assembly and run check_stream_kernel_assembly on it."""
+    """Compile the SpMV sources to assembly and run check_stream_kernel_assembly on each."""
+    checked = 0
     with tempfile.TemporaryDirectory() as tmp:
-        asm = os.path.join(tmp, "macko_spmv.s")
-        _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, "macko_spmv.hip"), "-o", asm],
-             verbose)
-        text = open(asm).read().splitlines()
-    return check_stream_kernel_assembly(text)
+        for source, (kernel_name, fixed_base, slot_registers) in TRACKED_KERNELS.items():
+            asm = os.path.join(tmp, source + ".s")
+            _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, source), "-o", asm], verbose)
+            with open(asm) as f:
+                checked += check_stream_kernel_assembly(f.read().splitlines(), kernel_name, fixed_base, slot_registers)
+    return checked
 
 
 def build_hip(verbose=False):
+    """Builds libmacko_hip.so.  The library only reaches its final path once the generated code
+    has passed the fixed-register check: an unchecked library must never be the one that loads."""
     out, _ = lib_paths()
+    verify_fixed_registers(verbose)
+    staging = out + ".building"
     cmd = [
         _hipcc(), *_DEVICE_FLAGS, "-fPIC", "-shared",
         *[os.path.join(_CSRC, s) for s in HIP_SOURCES],
-        "-o", out,
+        "-o", staging,
     ]
-    _run(cmd, verbose)
-    verify_fixed_registers(verbose)
+    try:
+        _run(cmd, verbose)
+        os.replace(staging, out)
+    finally:
+        if os.path.exists(staging):
+            os.remove(staging)
     return out
+
+
+STAMP = "macko_build.stamp"
+
+
+def source_digest():
+    """Hash of everything the two libraries are built from (csrc/, include/, this recipe)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    files = [os.path.abspath(__file__)]
+    for directory in (_CSRC, _INCLUDE):
+        files += [os.path.join(directory, name) for name in sorted(os.listdir(directory))]
+    for full in files:
+        if os.path.isfile(full):
+            h.update(os.path.basename(full).encode())
+            with open(full, "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def stamp_path():
+    return os.path.join(build_directory(), STAMP)
+
+
+def is_current():
+    """True when both libraries exist and were built from the sources as they are now."""
+    hip_lib, torch_lib = lib_paths()
+    if not (os.path.exists(hip_lib) and os.path.exists(torch_lib) and os.path.exists(stamp_path())):
+        return False
+    with open(stamp_path()) as f:
+        return f.read().strip() == source_digest()
 
 
 def build_torch(verbose=False):
@@ -166,7 +213,12 @@ def build_torch(verbose=False):
 
 
 def build_all(verbose=False):
-    return build_hip(verbose), build_torch(verbose)
+    if os.path.exists(stamp_path()):
+        os.remove(stamp_path())
+    built = build_hip(verbose), build_torch(verbose)
+    with open(stamp_path(), "w") as f:
+        f.write(source_digest() + "\n")
+    return built
 
 
 if __name__ == "__main__":

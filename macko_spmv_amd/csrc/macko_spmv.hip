@@ -19,216 +19,14 @@
 //
 // Behaviour restated from src/macko_spmv/cuda/kernels.cuh:34-124 of the upstream package.
 
-#include "macko_common.h"
+#include <atomic>
+
+#include "macko_spmv_detail.h"
 
 namespace macko {
 namespace {
 
-constexpr int kLdsFront = 16;   // zero bytes in front of x in LDS (masked head entries read here)
-constexpr int kLdsBack = 64;    // zero bytes behind x (masked tail entries read here)
-constexpr int kTileShift = 9;   // log2(kTile)
-constexpr int kXRegs = 2;       // 16-byte pieces of x a thread fetches with tracked loads
-
-struct SpmvArgs {
-    const u32 *values;      // fp16 pairs (or int8 quads for the int8 variant)
-    const u32 *deltas;      // 8 nibbles per word
-    const int *row_ptr;
-    const uint16_t *x;
-    uint16_t *y;
-    int rows;
-    int cols;
-    long long padded;       // P
-    float alpha;
-    float beta;
-    // Precomputed on the host so the kernel does no 64-bit division.  The P stored entries are
-    // dealt to the launch's W waves as evenly as possible: wave w starts at w*q + min(w, rem).
-    // Where wave w's first row should be if all rows were equally long, floor(w*rows/W), is
-    // w*rows_q + ((w*rows_frac) >> 32) with rows_frac = floor((rows % W) * 2^32 / W).
-    u32 entries_q, entries_rem;
-    u32 rows_q, rows_frac;
-    // 1 when there are no more rows than waves: wave w then simply owns rows
-    // [floor(w*rows/W), floor((w+1)*rows/W)), at most one row each.  No split of whole rows can do
-    // better than the longest row, and cutting by entries could hand one wave two rows.
-    u32 row_even;
-    // batched product (NB > 1 vectors per launch): elements between consecutive vectors of x / y
-    int ldx, ldy;
-    // fused x staging (XF != 0): the second operand of the function that produces x, and its epsilon
-    const uint16_t *x2;
-    float eps;
-#ifdef MACKO_SPMV_TRACE
-    long long *trace;  // 8 timestamps per wave (development builds only)
-#endif
-};
-
-#ifdef MACKO_SPMV_TRACE
-#define MACKO_STAMP(slot) \
-    do { if (a.trace && lane == 0) a.trace[(size_t)gw * 8 + (slot)] = (long long)__builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define MACKO_STAMP(slot) do { } while (0)
-#endif
-
-// First item of wave w when n items are dealt to the waves as evenly as possible.
-__device__ __forceinline__ u32 even_split(u32 w, u32 q, u32 rem) { return w * q + (w < rem ? w : rem); }
-
-__device__ __forceinline__ float half_bits_to_float(uint16_t h)
-{
-    return (float)__builtin_bit_cast(_Float16, h);
-}
-
-__device__ __forceinline__ uint16_t float_to_half_bits(float f)
-{
-    return __builtin_bit_cast(uint16_t, (_Float16)f);
-}
-
-// Where the first probe of the row search looks: 64 consecutive row_ptr values starting a few
-// rows before `guess`.
-__device__ __forceinline__ int probe_base(int guess, int rows)
-{
-    int w0 = guess - 8;
-    const int wmax = rows - 63;
-    w0 = w0 > wmax ? wmax : w0;
-    return w0 < 0 ? 0 : w0;
-}
-
-// Lane i of the returned value holds row_ptr[base + i] (row_ptr[rows] beyond the end).
-__device__ __forceinline__ int load_row_window(const int *__restrict__ row_ptr, int rows, int base, int lane)
-{
-    const int idx = base + lane;
-    return row_ptr[idx <= rows ? idx : rows];
-}
-
-// Smallest r in [0, rows] with row_ptr[r] >= target (rows if there is none), for two targets at
-// once.  All 64 lanes probe together.  window[k] is an already loaded probe (see
-// load_row_window) at base[k]; it resolves the search when rows carry similar entry counts.
-// Otherwise one more window is probed where the target should be if rows elsewhere are as long as
-// the ones just seen (which usually lands within a few rows even for very uneven matrices; that
-// window then replaces window[k] / base[k] so the caller finds its row starts in it), and 64-ary
-// rounds over what is still undecided follow.  Every value here is wave-uniform.
-__device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_ptr, int rows, int lane,
-                                                  const int target[2], int (&window)[2], int (&base)[2],
-                                                  int out[2])
-{
-    int lo[2], hi[2];
-    // narrows [lo, hi] with a window of row_ptr values: probed[i] >= target puts the answer at or
-    // before base + i, probed[i] < target puts it after
-    auto narrow = [&](int k, int probed, int at) {
-        const bool beyond = at + lane > rows;
-        const unsigned long long m = __ballot(beyond || probed >= target[k]);
-        if (m == 0) {
-            const int after = at + 64 > rows ? rows : at + 64;
-            lo[k] = lo[k] > after ? lo[k] : after;
-        } else {
-            const int f = __builtin_ctzll(m);
-            const int le = at + f > rows ? rows : at + f;
-            hi[k] = hi[k] < le ? hi[k] : le;
-            if (f > 0) lo[k] = lo[k] > le ? lo[k] : le;
-        }
-        if (lo[k] > hi[k]) lo[k] = hi[k];
-    };
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        lo[k] = 0;
-        hi[k] = rows;
-        narrow(k, window[k], base[k]);
-    }
-    if (__builtin_expect(lo[0] < hi[0] || lo[1] < hi[1], 0)) {
-        // second window, from the local row length: rows per entry around the first window
-        int probe[2], at[2];
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            at[k] = base[k];
-            if (lo[k] < hi[k]) {
-                const int last = base[k] + 63 <= rows ? 63 : rows - base[k];
-                const int v0 = __builtin_amdgcn_readlane(window[k], 0);
-                const int v1 = __builtin_amdgcn_readlane(window[k], last);
-                const float per_entry = (float)(last > 0 ? last : 1) / (float)(v1 > v0 ? v1 - v0 : 1);
-                float jump = (float)(target[k] - v0) * per_entry;
-                jump = jump > 2.0e9f ? 2.0e9f : (jump < -2.0e9f ? -2.0e9f : jump);
-                long long g = (long long)base[k] + (long long)jump - 32;
-                const int gmax = rows - 63 > 0 ? rows - 63 : 0;
-                g = g < lo[k] - 1 ? lo[k] - 1 : g;  // stay inside what is still undecided
-                g = g > hi[k] - 32 ? hi[k] - 32 : g;
-                g = g < 0 ? 0 : (g > gmax ? gmax : g);
-                at[k] = (int)g;
-            }
-            probe[k] = load_row_window(row_ptr, rows, at[k], lane);  // both loads in flight together
-        }
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            if (lo[k] < hi[k]) {
-                narrow(k, probe[k], at[k]);
-                window[k] = probe[k];
-                base[k] = at[k];
-            }
-        }
-    }
-    while (__builtin_expect(lo[0] < hi[0] || lo[1] < hi[1], 0)) {
-        int step[2], probe[2];
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            step[k] = (hi[k] - lo[k] + 63) >> 6;
-            const int idx = lo[k] + lane * step[k];
-            probe[k] = (lo[k] < hi[k] && idx < hi[k]) ? row_ptr[idx] : 0x7fffffff;
-        }
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            if (lo[k] < hi[k]) {
-                const unsigned long long m = __ballot(probe[k] >= target[k]);
-                if (m == 0) {
-                    lo[k] = lo[k] + 63 * step[k] + 1;
-                } else {
-                    const int f = __builtin_ctzll(m);
-                    const int at = lo[k] + f * step[k];
-                    if (f > 0) lo[k] = lo[k] + (f - 1) * step[k] + 1;
-                    if (at < hi[k]) hi[k] = at;
-                }
-                if (lo[k] > hi[k]) lo[k] = hi[k];
-            }
-        }
-    }
-    out[0] = lo[0];
-    out[1] = lo[1];
-}
-
-// Mask helpers: keep values [from, 8) / [0, upto) of a lane's 8 values (VB bytes each) and the
-// matching nibbles.  `from` / `upto` are wave-uniform, so the masks are built on the scalar unit.
-template <int VB>
-__device__ __forceinline__ void mask_from(u32x4 &v, u32 &d, int from)  // 1 <= from <= 7
-{
-    if (VB == 1) {  // 8 one-byte values in v.x, v.y
-        const unsigned long long m = ~0ull << (8 * from);
-        v.x &= (u32)m;
-        v.y &= (u32)(m >> 32);
-        d &= ~0u << (4 * from);
-        return;
-    }
-    const unsigned long long lo = from < 4 ? (~0ull << (16 * from)) : 0ull;
-    const unsigned long long hi = from < 4 ? ~0ull : (~0ull << (16 * (from - 4)));
-    v.x &= (u32)lo;
-    v.y &= (u32)(lo >> 32);
-    v.z &= (u32)hi;
-    v.w &= (u32)(hi >> 32);
-    d &= ~0u << (4 * from);
-}
-
-template <int VB>
-__device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= upto <= 7
-{
-    if (VB == 1) {
-        const unsigned long long m = (1ull << (8 * upto)) - 1;
-        v.x &= (u32)m;
-        v.y &= (u32)(m >> 32);
-        d &= (1u << (4 * upto)) - 1;
-        return;
-    }
-    const unsigned long long lo = upto < 4 ? ((1ull << (16 * upto)) - 1) : ~0ull;
-    const unsigned long long hi = upto <= 4 ? 0ull : ((1ull << (16 * (upto - 4))) - 1);
-    v.x &= (u32)lo;
-    v.y &= (u32)(lo >> 32);
-    v.z &= (u32)hi;
-    v.w &= (u32)(hi >> 32);
-    d &= (1u << (4 * upto)) - 1;
-}
+using namespace spmv_detail;
 
 // ---- loads whose completion is tracked by hand ---------------------------------------------
 // The tile ring, the row_ptr probe and the first pieces of x are fetched with inline-asm buffer
@@ -247,20 +45,6 @@ __device__ __forceinline__ void mask_upto(u32x4 &v, u32 &d, int upto)  // 1 <= u
 // v88.. ring: slot j keeps its values in v[88+4j : 91+4j] and its delta word in v[88+4D+j].
 
 constexpr int kCompilerVgprs = 78;
-constexpr u32 kNoTileValues = 0xfffff000u;  // beyond any values array (2P < 2^32 - 8192)
-constexpr u32 kNoTileDeltas = 0x7ffff000u;  // beyond any deltas array (P/2 < 2^30)
-
-__device__ __forceinline__ u32x4 make_buffer(const void *base, u32 bytes)
-{
-    const unsigned long long addr = reinterpret_cast<unsigned long long>(base);
-    u32x4 r;
-    r.x = uniform((int)(u32)addr);
-    r.y = uniform((int)((u32)(addr >> 32) & 0xffffu));
-    r.z = uniform((int)bytes);
-    r.w = 0x00020000u;
-    return r;
-}
-
 #define MACKO_FIXED_CLOBBERS_4 "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107"
 
 // row_ptr probe k (k = 0, 1) -> v78 + k
@@ -388,6 +172,9 @@ spmv_stream_kernel(const SpmvArgs a)
     u32 wg = blockIdx.x;
     if ((gridDim.x & 7) == 0) wg = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     const u32 gw = wg * WAVES + wave;
+#ifdef MACKO_DEV_HOOKS
+    const u32 stamp_wave = gw;
+#endif
     MACKO_STAMP(0);
 
 
@@ -702,13 +489,19 @@ spmv_stream_kernel(const SpmvArgs a)
     MACKO_STAMP(5);
 
     // The eight multiply-adds of a lane: entry k reads x at base + 2k + 2 * (nibbles 0..k), which is
-    // one v_dot8_u32_u4 with the multiplier 2 in the first k+1 nibble positions.
-    auto lane_fma = [&](const u32x4 &vv, u32 dd, u32 base) {
-        const u32 m[8] = {0x2u, 0x22u, 0x222u, 0x2222u, 0x22222u, 0x222222u, 0x2222222u, 0x22222222u};
+    // one v_dot8_u32_u4 with the multiplier 2 in the first k+1 nibble positions.  CHECKED (a piece
+    // of a row that ends inside the lane): entries kmax..7 of the lane are not part of the row;
+    // their value is masked to zero, but what they would read lies behind the row's last column
+    // and may be Inf or NaN, so they read the zero bytes in front of x instead.  (Entries in front
+    // of kmin, masked at a row's start, read those zero bytes by construction when x is in LDS.)
+    auto lane_fma = [&](const u32x4 &vv, u32 dd, u32 base, auto checked, int kmin, int kmax) {
+        constexpr bool CHECKED = decltype(checked)::value != 0;
+        const u32 zeros = row_origin - 16u;  // 16 zero bytes (times NB) in front of x
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const u32 addr = __builtin_amdgcn_udot8(dd, m[k], base, false);
-            if (NB > 1) {
+            u32 addr = __builtin_amdgcn_udot8(dd, twos_upto(k), base, false);
+            if constexpr (NB > 1) {
+                if (CHECKED) addr = k < kmax ? addr : zeros;
                 const u32 w = vv[k >> 1];
                 const float mv = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
                 const u32 at = x_addr + (addr << kBatchShift) + ((2 * k) << kBatchShift);
@@ -729,32 +522,30 @@ spmv_stream_kernel(const SpmvArgs a)
                     const uint16_t h = (b & 1) ? (uint16_t)(xs[b >> 1] >> 16) : (uint16_t)(xs[b >> 1] & 0xffffu);
                     accb[b] = __builtin_fmaf(mv, half_bits_to_float(h), accb[b]);
                 }
-                continue;
-            }
-            uint16_t xb;
-#if defined(MACKO_EXP_NO_GATHER)
-            xb = (uint16_t)(addr & 0x3fffu);
-#else
-            if (X_LDS) {
-                xb = *reinterpret_cast<lds_u16_ptr>((u32)(addr + 2 * k));  // ds_read_u16 with offset 2k
             } else {
-                int o = (int)(addr - x_addr) + 2 * k;
-                const int omax = 2 * a.cols - 2;
-                o = o < 0 ? 0 : (o > omax ? omax : o);
-                xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
+                uint16_t xb;
+                if (X_LDS) {
+                    if (CHECKED) addr = k < kmax ? addr : zeros;
+                    xb = *reinterpret_cast<lds_u16_ptr>((u32)(addr + 2 * k));  // ds_read_u16 with offset 2k
+                } else {
+                    int o = (int)(addr - x_addr) + 2 * k;
+                    const int omax = 2 * a.cols - 2;
+                    o = o < 0 ? 0 : (o > omax ? omax : o);
+                    if (CHECKED) o = (k >= kmin && k < kmax) ? o : 0x7ffffff0;  // past the end: reads as zero
+                    xb = __builtin_amdgcn_raw_buffer_load_b16(rs_x, o, 0, 0);
+                }
+                float m;
+                if (VB == 2) {
+                    const u32 w = vv[k >> 1];
+                    m = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+                } else {
+                    m = (float)((int)(vv[k >> 2] << (24 - 8 * (k & 3))) >> 24);  // sign-extended byte k
+                }
+                if (k & 1)
+                    acc1 = __builtin_fmaf(m, half_bits_to_float(xb), acc1);
+                else
+                    acc0 = __builtin_fmaf(m, half_bits_to_float(xb), acc0);
             }
-#endif
-            float m;
-            if (VB == 2) {
-                const u32 w = vv[k >> 1];
-                m = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
-            } else {
-                m = (float)((int)(vv[k >> 2] << (24 - 8 * (k & 3))) >> 24);  // sign-extended byte k
-            }
-            if (k & 1)
-                acc1 = __builtin_fmaf(m, half_bits_to_float(xb), acc1);
-            else
-                acc0 = __builtin_fmaf(m, half_bits_to_float(xb), acc0);
         }
     };
 
@@ -762,25 +553,17 @@ spmv_stream_kernel(const SpmvArgs a)
     // advances the row address by 16 bytes (its 8 entries) plus twice its nibble sum; the DPP scan
     // of that quantity gives every lane its starting address.
     auto full_tile_pass = [&](const u32x4 &vj, u32 dj) {
-#if defined(MACKO_EXP_NO_COMPUTE)
-        acc0 += __builtin_bit_cast(float, (vj.x ^ vj.y ^ vj.z ^ vj.w ^ dj) & 0x3fffffffu);
-        return;
-#endif
         const u32 step = __builtin_amdgcn_udot8(dj, 0x22222222u, 16u, false);
         const u32 incl = (u32)wave_scan_inclusive((int)step);
         const u32 base = (incl - step) + row_addr;
         row_addr += (u32)__builtin_amdgcn_readlane((int)incl, kWave - 1);
-        lane_fma(vj, dj, base);
+        lane_fma(vj, dj, base, index_constant<0>{}, 0, 8);
     };
 
     // Entries [pos, seg_end) of the tile starting at entry `tb`, all in the current row: lanes
     // outside the segment are switched off, the first and last lane of the segment are masked.
     // A row that starts `q0` entries into its first lane shifts every address by -2*q0.
     auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end) {
-#if defined(MACKO_EXP_NO_COMPUTE)
-        acc0 += __builtin_bit_cast(float, (vj.x ^ vj.y ^ vj.z ^ vj.w ^ dj) & 0x3fffffffu);
-        return;
-#endif
         const int rel0 = pos - tb;
         const int rel1 = seg_end - tb;
         const int l0 = rel0 >> 3, q0 = rel0 & 7;
@@ -796,7 +579,13 @@ spmv_stream_kernel(const SpmvArgs a)
         const u32 origin = row_addr - 2u * (u32)q0;
         const u32 base = (incl - step) + origin;
         row_addr = origin + (u32)__builtin_amdgcn_readlane((int)incl, kWave - 1);
-        if (active) lane_fma(vv, dd, base);
+        const int kmin = lane == l0 ? q0 : 0;
+        const int kmax = (lane == l1 && q1 != 0) ? q1 : 8;
+#ifdef MACKO_NO_CHECK
+        if (active) lane_fma(vv, dd, base, index_constant<0>{}, kmin, kmax);
+#else
+        if (active) lane_fma(vv, dd, base, index_constant<1>{}, kmin, kmax);
+#endif
     };
 
     auto finish_row = [&]() {
@@ -873,33 +662,37 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
     a.rows_frac = (u32)(((unsigned long long)((u32)a.rows % n_waves) << 32) / n_waves);
     a.row_even = (u32)a.rows <= n_waves ? 1u : 0u;
     if (lds_bytes > 64 * 1024) {
-        // one-time opt-in to more than 64 KiB of dynamic LDS, per device
-        static bool done[64] = {};
+        // one-time opt-in to more than 64 KiB of dynamic LDS, per device and kernel
+        static std::atomic<bool> done[64];
         int dev = 0;
         hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return (int)e;
-        if (dev < 0 || dev >= 64 || !done[dev]) {
+        if (dev < 0 || dev >= 64 || !done[dev].load(std::memory_order_acquire)) {
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return (int)e;
-            if (dev >= 0 && dev < 64) done[dev] = true;
+            if (dev >= 0 && dev < 64) done[dev].store(true, std::memory_order_release);
         }
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(BLOCK), lds_bytes, stream, a);
     return (int)hipGetLastError();
 }
 
-// Launch-shape overrides for tuning runs (0 = built-in default).  Not part of the public ABI.
+#ifdef MACKO_DEV_HOOKS
+// Launch-shape overrides for tuning runs (0 = built-in default); development builds only.
 struct Tuning {
-    int block;      // threads per workgroup: 256, 512 or 1024
-    int depth;      // tiles in flight per wave: 1, 2 or 4 (4 only with 1024 threads, 1 only with 1024)
-    int wg_per_cu;  // workgroups launched per compute unit
+    int depth;  // tiles in flight per wave: 1 or 2
+    int grid;   // workgroups
+    int split;  // 1: always the split kernel, -1: never
 };
 Tuning g_tuning = {0, 0, 0};
+long long *g_trace = nullptr;
+#endif
 
 template <bool AXPBY, int VB = 2, int NB = 1, int XF = 0>
-int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
+int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
 {
+    SpmvArgs a = args;
     if (a.rows == 0) return 0;
     if (a.padded == 0) {
         hipLaunchKernelGGL(spmv_empty_kernel<AXPBY>, dim3((a.rows + 255) / 256), dim3(256), 0, stream, a.y,
@@ -910,10 +703,7 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     int rc = device_info(&info);
     if (rc != 0) return rc;
 
-    const Tuning t = g_tuning;
-    const int block = t.block ? t.block : 1024;
-    const int wg_per_cu = t.wg_per_cu ? t.wg_per_cu : 1;
-    const int waves = block / kWave;
+    constexpr int waves = 1024 / kWave;
     // about one wave per tile at most, so tiny matrices get a small grid; but when rows are about
     // a tile long, prefer one wave per row over a slightly smaller wave count that would leave
     // some waves with two rows
@@ -921,46 +711,58 @@ int spmv_dispatch(const SpmvArgs &a, hipStream_t stream)
     long long waves_wanted = n_tiles;
     if (a.rows > waves_wanted) waves_wanted = a.rows < 2 * n_tiles ? a.rows : 2 * n_tiles;
     long long grid = (waves_wanted + waves - 1) / waves;
-    if (grid > (long long)info.compute_units * wg_per_cu) grid = (long long)info.compute_units * wg_per_cu;
+    if (grid > (long long)info.compute_units) grid = (long long)info.compute_units;
     if (grid < 1) grid = 1;
+    // Whole rows per wave need about as many rows as waves; with clearly fewer, the workgroups own
+    // the rows and their waves split them (macko_spmv_split.hip): one workgroup per compute unit,
+    // at least a tile per wave and a row per workgroup.
+    // Only where rows are long (four tiles and more on average): for short rows a wave per row is
+    // the cheaper way even if most waves stay idle.
+    bool split = 4 * (long long)a.rows < 3 * grid * waves && n_tiles >= 4 * (long long)a.rows;
+#ifdef MACKO_DEV_HOOKS
+    if (g_tuning.split) split = g_tuning.split > 0;
+    a.trace = g_trace;
+#endif
+    const size_t lds_x = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack) + (XF == 1 ? 64 : 0);
+    constexpr size_t piece_bytes = (size_t)waves * 4 * (NB + 1) + 4;  // what the split kernel keeps behind x
+    if (split) {
+        long long grid_split = (n_tiles + waves - 1) / waves;
+        if (grid_split > a.rows) grid_split = a.rows;
+        if (grid_split > (long long)info.compute_units) grid_split = (long long)info.compute_units;
+        if (grid_split < 1) grid_split = 1;
+#ifdef MACKO_DEV_HOOKS
+        if (g_tuning.grid) grid_split = g_tuning.grid;
+#endif
+        const bool fits = lds_x + piece_bytes <= (size_t)info.max_lds_bytes;
+        if (!fits && (XF != 0 || NB > 1)) return MACKO_E_INVALID_ARGUMENT;
+        return spmv_split_launch(a, AXPBY, VB, NB, XF, fits, (int)grid_split, fits ? lds_x : 0, stream);
+    }
     // Ring depth: one tile in flight behind the one being processed is enough, and cheapest to
     // start, when a wave walks only a few tiles; from about four tiles per wave on, two do better
     // (measured on the Llama shapes and larger ones, fp16 and int8; deeper is slower).
-    const long long n_waves = grid * waves;
-    const int depth = t.depth ? t.depth : (n_tiles >= 4 * n_waves ? 2 : 1);
-
-    const size_t lds_need = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack) + (XF == 1 ? 64 : 0);
+    int depth = n_tiles >= 4 * grid * waves ? 2 : 1;
+#ifdef MACKO_DEV_HOOKS
+    if (g_tuning.depth) depth = g_tuning.depth;
+    if (g_tuning.grid) grid = g_tuning.grid;
+#endif
+    const bool fits = lds_x <= (size_t)info.max_lds_bytes;
     if (XF != 0) {  // fused staging: x must fit in LDS (checked by the caller too)
-        if (lds_need > (size_t)info.max_lds_bytes || block != 1024) return MACKO_E_INVALID_ARGUMENT;
-        if (depth == 2) return launch_stream<1024, 2, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_need, stream);
-        return launch_stream<1024, 1, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_need, stream);
+        if (!fits) return MACKO_E_INVALID_ARGUMENT;
+        if (depth == 2) return launch_stream<1024, 2, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_x, stream);
+        return launch_stream<1024, 1, true, AXPBY, 2, 1, XF>(a, (int)grid, lds_x, stream);
     }
     if (NB > 1) {  // NB vectors per launch: the caller has checked that they fit in LDS
-        if (lds_need > (size_t)info.max_lds_bytes || block != 1024) return MACKO_E_INVALID_ARGUMENT;
-        if (depth == 2) return launch_stream<1024, 2, true, false, 2, NB>(a, (int)grid, lds_need, stream);
-        return launch_stream<1024, 1, true, false, 2, NB>(a, (int)grid, lds_need, stream);
+        if (!fits) return MACKO_E_INVALID_ARGUMENT;
+        if (depth == 2) return launch_stream<1024, 2, true, false, 2, NB>(a, (int)grid, lds_x, stream);
+        return launch_stream<1024, 1, true, false, 2, NB>(a, (int)grid, lds_x, stream);
     }
-    if (lds_need > (size_t)info.max_lds_bytes)
-        return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
-    if (VB == 1) {  // int8 values: the default launch shapes only
-        if (block == 1024 && depth == 2)
-            return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_need, stream);
-        if (block == 1024 && depth == 1)
-            return launch_stream<1024, 1, true, AXPBY, VB>(a, (int)grid, lds_need, stream);
-        return MACKO_E_INVALID_ARGUMENT;
-    }
-#define MACKO_CASE(B, D_) \
-    if (block == B && depth == D_) return launch_stream<B, D_, true, AXPBY>(a, (int)grid, lds_need, stream);
-    MACKO_CASE(1024, 2)
-    MACKO_CASE(1024, 1)
-    if (!AXPBY) {  // the other shapes exist for tuning runs of the plain product only
-        MACKO_CASE(1024, 4)
-        MACKO_CASE(512, 2)
-        MACKO_CASE(256, 2)
-    }
-#undef MACKO_CASE
-    return MACKO_E_INVALID_ARGUMENT;
+    if (!fits) return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
+    if (depth == 2) return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
+    return launch_stream<1024, 1, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
 }
+
+// LDS the split kernel keeps behind x at most (16 waves, up to 8 vectors and a flag each)
+constexpr size_t kSplitPieceBytes = 16 * 4 * 9 + 4;
 
 int check_spmv_args(const void *values, const void *deltas, const int32_t *row_ptr, const void *x, void *y,
                     int32_t rows, int32_t cols, int64_t padded, int value_bytes = 2)
@@ -982,16 +784,14 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 }  // namespace
 }  // namespace macko
 
-#ifdef MACKO_SPMV_TRACE
-static long long *g_trace = nullptr;
-extern "C" void macko_spmv_set_trace(long long *device_buffer) { g_trace = device_buffer; }
-#endif
-
-// Tuning hook used by benchmark sweeps; see struct Tuning.
-extern "C" void macko_spmv_tune(int block, int depth, int wg_per_cu)
+#ifdef MACKO_DEV_HOOKS
+extern "C" void macko_spmv_set_trace(long long *device_buffer) { macko::g_trace = device_buffer; }
+extern "C" void macko_spmv_tune(int depth, int grid, int active, int split)
 {
-    macko::g_tuning = macko::Tuning{block, depth, wg_per_cu};
+    (void)active;
+    macko::g_tuning = macko::Tuning{depth, grid, split};
 }
+#endif
 
 extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_ptr, const void *x,
                               void *y, int32_t rows, int32_t cols, int64_t padded_entries, void *stream)
@@ -1003,9 +803,6 @@ extern "C" int macko_spmv_f16(const void *values, const void *deltas, const int3
                rows,                cols,                padded_entries, 1.0f,          0.0f,
                0,                   0,                   0,              0,             0,
                0,                   0};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = g_trace;
-#endif
     return spmv_dispatch<false>(a, as_stream(stream));
 }
 
@@ -1020,9 +817,6 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
                rows,                cols,                padded_entries, alpha,         beta,
                0,                   0,                   0,              0,             0,
                0,                   0};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = nullptr;
-#endif
     return spmv_dispatch<true>(a, as_stream(stream));
 }
 
@@ -1037,9 +831,6 @@ extern "C" int macko_spmv_i8f16(const void *values, const void *deltas, const in
                rows,                cols,                padded_entries, 1.0f,          0.0f,
                0,                   0,                   0,              0,             0,
                0,                   0};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = nullptr;
-#endif
     return spmv_dispatch<false, 1>(a, as_stream(stream));
 }
 
@@ -1054,9 +845,6 @@ extern "C" int macko_spmv_i8f16_axpby(const void *values, const void *deltas, co
                rows,                cols,                padded_entries, alpha,         beta,
                0,                   0,                   0,              0,             0,
                0,                   0};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = nullptr;
-#endif
     return spmv_dispatch<true, 1>(a, as_stream(stream));
 }
 
@@ -1086,17 +874,14 @@ extern "C" int macko_spmv_f16_batched(const void *values, const void *deltas, co
         SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr,
                    (const uint16_t *)x + (size_t)done * (size_t)ldx, (uint16_t *)y + (size_t)done * (size_t)ldy,
                    rows, cols, padded_entries, 1.0f, 0.0f, 0, 0, 0, 0, 0, (int)ldx, (int)ldy};
-#ifdef MACKO_SPMV_TRACE
-        a.trace = nullptr;
-#endif
         int step;
-        if (padded_entries > 0 && left >= 8 && 8 * per_vector <= (size_t)info.max_lds_bytes) {
+        if (padded_entries > 0 && left >= 8 && 8 * per_vector + kSplitPieceBytes <= (size_t)info.max_lds_bytes) {
             step = 8;
             rc = spmv_dispatch<false, 2, 8>(a, as_stream(stream));
-        } else if (padded_entries > 0 && left >= 4 && 4 * per_vector <= (size_t)info.max_lds_bytes) {
+        } else if (padded_entries > 0 && left >= 4 && 4 * per_vector + kSplitPieceBytes <= (size_t)info.max_lds_bytes) {
             step = 4;
             rc = spmv_dispatch<false, 2, 4>(a, as_stream(stream));
-        } else if (padded_entries > 0 && left >= 2 && 2 * per_vector <= (size_t)info.max_lds_bytes) {
+        } else if (padded_entries > 0 && left >= 2 && 2 * per_vector + kSplitPieceBytes <= (size_t)info.max_lds_bytes) {
             step = 2;
             rc = spmv_dispatch<false, 2, 2>(a, as_stream(stream));
         } else {
@@ -1120,7 +905,7 @@ int check_fused_args(const void *x, const void *x2, int32_t cols, int64_t padded
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != 0) return rc;
-    if ((size_t)kLdsFront + 2 * (size_t)cols + kLdsBack + 64 > (size_t)info.max_lds_bytes) return MACKO_E_INVALID_ARGUMENT;
+    if ((size_t)kLdsFront + 2 * (size_t)cols + kLdsBack + 64 + kSplitPieceBytes > (size_t)info.max_lds_bytes) return MACKO_E_INVALID_ARGUMENT;
     return 0;
 }
 }  // namespace
@@ -1141,9 +926,6 @@ extern "C" int macko_spmv_f16_rmsnorm(const void *values, const void *deltas, co
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)x, (uint16_t *)y,
                rows, cols, padded_entries, 1.0f, 0.0f, 0, 0, 0, 0, 0, 0, 0, (const uint16_t *)norm_weight, eps};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = nullptr;
-#endif
     return spmv_dispatch<false, 2, 1, 1>(a, as_stream(stream));
 }
 
@@ -1161,9 +943,6 @@ extern "C" int macko_spmv_f16_silu_mul_axpby(const void *values, const void *del
     if (rc != 0) return rc;
     SpmvArgs a{(const u32 *)values, (const u32 *)deltas, row_ptr, (const uint16_t *)gate, (uint16_t *)y,
                rows, cols, padded_entries, alpha, beta, 0, 0, 0, 0, 0, 0, 0, (const uint16_t *)up, 0.0f};
-#ifdef MACKO_SPMV_TRACE
-    a.trace = nullptr;
-#endif
     if (beta == 0.0f && alpha == 1.0f) return spmv_dispatch<false, 2, 1, 2>(a, as_stream(stream));
     return spmv_dispatch<true, 2, 1, 2>(a, as_stream(stream));
 }
