@@ -1,22 +1,29 @@
 #!/usr/bin/env python3
 """Single-GPU benchmark of the MACKO SpMV path on MI355X.
 
-Workload (`config.workload`): the Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as
-fp16 SpMV, weights N(0, 0.02) pruned per output row to density d in {0.1,0.2,0.3,0.5,0.7,0.9}
-(keep the round(d*cols) largest |w| of each row), x ~ N(0,1) fp16.  One "step" is one multiply of
-every (shape, density) pair: 18 kernel launches.  Steps are replayed from a HIP graph so the GPU
-is not waiting for Python between launches; two copies of every matrix alternate, and one step
-streams about 0.7 GB, so nothing is served from the 256 MB last-level cache.
+Headline workload (`config.workload`, `value`, `roofline`): the Llama-2-7B layer shapes 4096x4096,
+11008x4096, 4096x11008 as fp16 SpMV, weights N(0, 0.02) pruned per output row to density d in
+{0.1,0.2,0.3,0.5,0.7,0.9} (keep the round(d*cols) largest |w| of each row), x ~ N(0,1) fp16.  One
+"step" is one multiply of every (shape, density) pair: 18 kernel launches.  Steps are replayed from
+a HIP graph so the GPU is not waiting for Python between launches; two copies of every matrix
+alternate, and one step streams about 0.7 GB, so nothing is served from the 256 MB last-level cache.
+
+The same run also measures, each the same way and reported under `suites`: the large LLM shapes
+with Bernoulli masks, the skewed-row stress matrix, and shapes with fewer rows than the GPU has
+waves.
 
 Reported: effective HBM bandwidth = algorithmic bytes / time with
     bytes = 2*P (values) + P/2 (deltas) + 4*(R+1) (row_ptr) + 2*C (x) + 2*R (y),
-P = stored entries incl. padding, against the 8 TB/s peak; per-case times and the speed-up over
-torch's dense fp16 GEMV measured the same way; and a single-thread CPU baseline (the C restatement
-of the upstream CPU path) on a bounded sample.
+P = stored entries incl. padding, against the 8 TB/s peak; per-case times, the time a kernel needs
+that only reads the same number of bytes, and the speed-up over torch's dense fp16 GEMV measured
+the same way; and the CPU route (compress, then a dense fp32 product on the host) on a bounded
+sample.
 
 Prints ONE JSON line on stdout; progress goes to stderr.
 """
 import argparse
+import ctypes
+import gc
 import json
 import os
 import sys
@@ -31,12 +38,13 @@ SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008)]
 DENSITIES = [0.1, 0.2, 0.3, 0.5, 0.7, 0.9]
 LARGE_SHAPES = [(28672, 8192), (8192, 28672), (12288, 49152), (49152, 12288)]
 LARGE_DENSITIES = [0.1, 0.3, 0.5]
+FEW_ROW_SHAPES = [(1024, 8192), (512, 16384), (64, 49152)]
+FEW_ROW_DENSITIES = [0.1, 0.5]
 
-# HBM bytes per launch of spmv_stream_kernel, averaged over the 18 launches of one step of the
-# default workload: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, each scaled by what the
-# same counter reports for calibration_copy_kernel on 256 MiB (factors 0.5000 and 1.0000).  Source:
-# profiles/spmv_stream_kernel_llama_shapes_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama": 40.80e6}
+# HBM bytes per launch measured with rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by
+# what the same counter reads for a copy of known size); recorded per suite, with the commit they
+# were measured at, in this file.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 WORKLOADS = {
     "llama": "configs[1]: Llama-2-7B layer shapes 4096x4096, 11008x4096, 4096x11008 as fp16 SpMV, per-row "
@@ -48,6 +56,9 @@ WORKLOADS = {
     "skew": "configs[3]: 14336x4096 fp16, per-row density from a power law (alpha 1.5) clipped to [0.01, 0.95] "
             "with mean 0.3, all-zero rows and a 40-column zero gap in every row, next to a uniform Bernoulli "
             "0.3 matrix of the same shape; one step = one multiply of each, replayed from a HIP graph",
+    "fewrows": "matrices with fewer rows than the GPU has waves (1024x8192, 512x16384, 64x49152; Bernoulli "
+               "masks at density 0.1 and 0.5): rows are split between the waves of a workgroup; one step = one "
+               "multiply of each of the 6 pairs, replayed from a HIP graph",
 }
 
 
@@ -61,6 +72,18 @@ def algorithmic_bytes(P, rows, cols):
 
 def dense_bytes(rows, cols):
     return 2 * rows * cols + 2 * cols + 2 * rows
+
+
+def load_traffic(suite):
+    """(HBM bytes per launch, where the figure comes from) for a suite, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(suite)
+    except (OSError, ValueError):
+        return None, None
+    if not entry:
+        return None, None
+    return entry.get("hbm_bytes_per_launch"), f"{entry.get('source')} (measured at commit {entry.get('commit')})"
 
 
 def make_pruned(torch, rows, cols, density, seed):
@@ -106,23 +129,34 @@ def make_skewed(torch, rows, cols, seed, mean_density=0.3, alpha=1.5, lo=0.01, h
     return W.contiguous(), x
 
 
-def make_inputs(torch, suite):
-    """List of (rows, cols, label, W, x) for a workload."""
+def input_specs(suite):
+    """List of (rows, cols, label, maker) for a workload; maker(torch) -> (W, x)."""
     out = []
     if suite == "llama":
         for si, (rows, cols) in enumerate(SHAPES):
             for di, d in enumerate(DENSITIES):
-                out.append((rows, cols, d, *make_pruned(torch, rows, cols, d, seed=1000 * si + di)))
+                out.append((rows, cols, d, lambda t, r=rows, c=cols, d=d, s=1000 * si + di: make_pruned(t, r, c, d, s)))
     elif suite == "large":
         for si, (rows, cols) in enumerate(LARGE_SHAPES):
             for di, d in enumerate(LARGE_DENSITIES):
-                out.append((rows, cols, d, *make_bernoulli(torch, rows, cols, d, seed=5000 + 100 * si + di)))
+                out.append((rows, cols, d,
+                            lambda t, r=rows, c=cols, d=d, s=5000 + 100 * si + di: make_bernoulli(t, r, c, d, s)))
     elif suite == "skew":
-        out.append((14336, 4096, "skewed", *make_skewed(torch, 14336, 4096, seed=9000)))
-        out.append((14336, 4096, 0.3, *make_bernoulli(torch, 14336, 4096, 0.3, seed=9001)))
+        out.append((14336, 4096, "skewed", lambda t: make_skewed(t, 14336, 4096, seed=9000)))
+        out.append((14336, 4096, 0.3, lambda t: make_bernoulli(t, 14336, 4096, 0.3, seed=9001)))
+    elif suite == "fewrows":
+        for si, (rows, cols) in enumerate(FEW_ROW_SHAPES):
+            for di, d in enumerate(FEW_ROW_DENSITIES):
+                out.append((rows, cols, d,
+                            lambda t, r=rows, c=cols, d=d, s=7000 + 100 * si + di: make_bernoulli(t, r, c, d, s)))
     else:
         raise ValueError(suite)
     return out
+
+
+def make_inputs(torch, suite):
+    """List of (rows, cols, label, W, x) for a workload (all matrices at once: small suites only)."""
+    return [(rows, cols, d, *maker(torch)) for rows, cols, d, maker in input_specs(suite)]
 
 
 def clone_compressed(c):
@@ -152,112 +186,53 @@ def time_graph(torch, fn, replays):
     return start.elapsed_time(end) * 1e-3 / replays, graph
 
 
-def cpu_baseline(torch, sample):
-    """Time the C restatement of the upstream CPU path (single thread) on `sample` cases."""
-    import numpy as np
+class ReadYardstick:
+    """Time of a kernel that only reads a given number of bytes (one launch, rotating through a pool
+    larger than the last-level cache): what any one-launch kernel needs just to pull them out of HBM."""
 
-    from oracle import macko_oracle as mo
+    WHAT = ("calibration_read_kernel: one launch that only reads the same number of bytes (256x1024 threads, "
+            "contiguous span per wave, four non-temporal 16-byte loads per lane in flight), timed like the "
+            "per-case SpMV figures")
 
-    t_compress = t_spmv = t_dense = 0.0
-    total_bytes = 0
-    for W, x, _ in sample:
-        dense = W.cpu().numpy()
-        xs = x.cpu().numpy()
-        t0 = time.perf_counter()
-        values, deltas, row_ptr, n = mo.compress(dense)
-        t1 = time.perf_counter()
-        y = mo.spmv(values, deltas, row_ptr, dense.shape[0], dense.shape[1], xs)
-        t2 = time.perf_counter()
-        yd = mo.dense_gemv(dense, xs)
-        t3 = time.perf_counter()
-        assert np.allclose(y.view(np.float16).astype(np.float32), yd.view(np.float16).astype(np.float32),
-                           rtol=1e-2, atol=1e-3)
-        # the compressor walks the matrix twice in this wrapper (count, then fill): report one walk
-        t_compress += (t1 - t0) / 2
-        t_spmv += t2 - t1
-        t_dense += t3 - t2
-        total_bytes += algorithmic_bytes(values.size, dense.shape[0], dense.shape[1])
-    return {
-        "value": round(total_bytes / t_spmv / 1e9, 3),
-        "unit": "GB/s",
-        "cores": 1,
-        "kind": "port",
-        "sample": "one SpMV each of 4096x4096, 11008x4096, 4096x11008 at density 0.5 from the compressed "
-                  "arrays (C restatement of the upstream decode + fp32 accumulate, scalar, 1 thread)",
-        "spmv_s": round(t_spmv, 4),
-        "compress_s": round(t_compress, 4),
-        "dense_fp32_matvec_s": round(t_dense, 4),
-        "host_cpus": os.cpu_count(),
-    }
+    def __init__(self, torch, bench_lib, largest_bytes):
+        self.torch = torch
+        self.lib = bench_lib
+        # the pool holds at least two copies of the largest case, so consecutive launches never re-read
+        self.pool_bytes = max(1 << 30, 2 * self.stride(largest_bytes))
+        self.pool = torch.ones(self.pool_bytes, dtype=torch.uint8, device="cuda")
+        self.sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    @staticmethod
+    def stride(nbytes):
+        return (int(nbytes) // 16 * 16 + 4095) // 4096 * 4096
+
+    def seconds(self, nbytes, replays):
+        nbytes = int(nbytes) // 16 * 16
+        stride = self.stride(nbytes)
+        copies = self.pool_bytes // stride
+
+        def launches():
+            sp = self.torch.cuda.current_stream().cuda_stream
+            for k in range(copies):
+                assert k * stride + nbytes <= self.pool_bytes  # the kernel trusts its arguments
+                rc = self.lib.macko_calibration_read(self.pool.data_ptr() + k * stride, nbytes, self.sink.data_ptr(), sp)
+                assert rc == 0, rc
+
+        t, _ = time_graph(self.torch, launches, replays)
+        return t / copies
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
-    ap.add_argument("--no-compress", action="store_true", help="skip the compressor timing")
-    ap.add_argument("--no-int8", action="store_true", help="skip the int8-values variant timing")
-    ap.add_argument("--no-batched", action="store_true", help="skip the batched-product timing")
-    ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
-    ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
-                    help="llama = the headline workload; large / skew = the other shape families")
-    ap.add_argument("--calibration-copies", type=int, default=0,
-                    help="also launch calibration_copy_kernel on a 256 MiB buffer this many times "
-                         "(reference dispatches for scaling rocprofv3 byte counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (rows would shard across GPUs, but no "
-                 "multi-GPU path is part of it); run with --gpus 1")
+def load_bench_library():
+    from macko_spmv_amd import _build
 
-    import torch
+    lib = ctypes.CDLL(_build.bench_lib_path())
+    lib.macko_calibration_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    lib.macko_calibration_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    return lib
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible; the MACKO path has no CPU implementation to benchmark")
-    import macko_spmv_amd as mk
 
-    dev = torch.cuda.get_device_properties(0)
-    log(f"device: {dev.name}, {dev.multi_processor_count} CUs")
-
-    # ---- inputs ---------------------------------------------------------------------------------
-    cases = []
-    for rows, cols, d, W, x in make_inputs(torch, args.suite):
-        c = mk.compress(W)
-        P = c[0].numel()
-        cases.append({"rows": rows, "cols": cols, "density": d, "P": P, "x": x,
-                      "copies": [c, clone_compressed(c)], "W": W,
-                      "bytes": algorithmic_bytes(P, rows, cols)})
-        log(f"case {rows}x{cols} d={d}: P={P} bytes={cases[-1]['bytes'] / 1e6:.1f} MB")
-    step_bytes = sum(c["bytes"] for c in cases)
-    n_launch = len(cases)
-
-    # correctness of what is about to be timed (cheap: one case per shape, fp32 dense product)
-    for c in cases[3::6] if args.suite == "llama" else cases:
-        y = mk.multiply(c["copies"][0], c["x"]).float()
-        want = c["W"].float() @ c["x"].float()
-        assert torch.allclose(y, want, rtol=1e-2, atol=1e-3), "multiply disagrees with the dense product"
-
-    if args.calibration_copies > 0:
-        import ctypes
-
-        lib = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
-        lib.macko_calibration_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
-        n_bytes = 256 << 20
-        src = torch.ones(n_bytes // 2, dtype=torch.float16, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(args.calibration_copies):
-            rc = lib.macko_calibration_copy(src.data_ptr(), dst.data_ptr(), n_bytes,
-                                            torch.cuda.current_stream().cuda_stream)
-            assert rc == 0, rc
-        torch.cuda.synchronize()
-        assert torch.equal(src, dst)
-        log(f"calibration: {args.calibration_copies} copies of {n_bytes} bytes "
-            f"(each reads {n_bytes} and writes {n_bytes} bytes)")
-        del src, dst
-
-    # ---- the timed region: K steps replayed from graphs on a side stream --------------------------
+def timed_steps(torch, mk, cases, steps, warmup):
+    """K steps replayed from graphs on a side stream; returns seconds for exactly `steps` steps."""
     def step(copy):
         for c in cases:
             mk.multiply(c["copies"][copy], c["x"])
@@ -277,89 +252,257 @@ def main():
         g1 = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g1, stream=stream):
             step(0)
-        for _ in range(args.warmup // 2):
+        for _ in range(warmup // 2):
             g2.replay()
-        if args.warmup % 2:
+        if warmup % 2:
             g1.replay()
         stream.synchronize()
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         start.record(stream)
-        for _ in range(args.steps // 2):
+        for _ in range(steps // 2):
             g2.replay()
-        if args.steps % 2:
+        if steps % 2:
             g1.replay()
         end.record(stream)
         end.synchronize()
         torch.cuda.synchronize()
-    elapsed_s = start.elapsed_time(end) * 1e-3
-    ms_per_step = elapsed_s * 1e3 / args.steps
-    gbps = step_bytes * args.steps / elapsed_s / 1e9
-    launch_us = elapsed_s * 1e6 / (args.steps * n_launch)
-    log(f"timed region: {args.steps} steps, {ms_per_step:.4f} ms/step, {gbps:.1f} GB/s effective, "
+    torch.cuda.current_stream().wait_stream(stream)
+    return start.elapsed_time(end) * 1e-3
+
+
+def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with_dense=True, keep_dense=False):
+    """Builds a workload, checks what is about to be timed against the dense product, times `steps`
+    steps of it and every case on its own.  Returns (summary dict, cases) -- `cases` keep their
+    inputs only when keep_dense is set."""
+    cases = []
+    for rows, cols, d, maker in input_specs(suite):
+        W, x = maker(torch)
+        c = mk.compress(W)
+        P = c[0].numel()
+        case = {"rows": rows, "cols": cols, "density": d, "P": P, "x": x, "copies": [c, clone_compressed(c)],
+                "bytes": algorithmic_bytes(P, rows, cols)}
+        # correctness of what is about to be timed: the dense fp32-accumulated product, every case
+        y = mk.multiply(c, x).float()
+        want = W.float() @ x.float()
+        assert torch.allclose(y, want, rtol=1e-2, atol=1e-3), f"multiply disagrees with the dense product ({suite} {rows}x{cols} d={d})"
+        del y, want
+        per = {"shape": f"{rows}x{cols}", "density": d}
+        if with_dense:
+            # dense baselines now, while W is at hand: W @ x as in the upstream script, and the same
+            # product phrased as a one-row GEMM, which hipBLASLt serves with other kernels
+            db = dense_bytes(rows, cols)
+            n_dense = max(2, min(64, int(1.0e9 // db) + 1))
+            dense_copies = [W] + [W.clone() for _ in range(n_dense - 1)]
+            t_dense, _ = time_graph(torch, lambda: [torch.matmul(Wc, x) for Wc in dense_copies], case_replays)
+            x_row = x[None, :]
+            t_gemm, _ = time_graph(torch, lambda: [torch.matmul(x_row, Wc.t()) for Wc in dense_copies], case_replays)
+            per["dense_us"] = round(t_dense / n_dense * 1e6, 2)
+            per["dense_as_gemm_us"] = round(t_gemm / n_dense * 1e6, 2)
+            per["dense_gbps"] = round(db / (t_dense / n_dense) / 1e9, 1)
+            del dense_copies
+        case["per"] = per
+        if keep_dense:
+            case["W"] = W
+        del W
+        cases.append(case)
+        log(f"[{suite}] case {rows}x{cols} d={d}: P={P} bytes={case['bytes'] / 1e6:.1f} MB")
+    step_bytes = sum(c["bytes"] for c in cases)
+    n_launch = len(cases)
+
+    elapsed_s = timed_steps(torch, mk, cases, steps, warmup)
+    gbps = step_bytes * steps / elapsed_s / 1e9
+    launch_us = elapsed_s * 1e6 / (steps * n_launch)
+    log(f"[{suite}] timed region: {steps} steps, {elapsed_s * 1e3 / steps:.4f} ms/step, {gbps:.1f} GB/s effective, "
         f"{launch_us:.2f} us per launch on average")
 
-    # ---- per-case timing, MACKO and dense, each over >= 1 GB of distinct copies ------------------
+    # per-case timing, each over >= 1 GB of distinct copies
     per_case = []
-    if not args.no_dense:
-        import ctypes
+    for c in cases:
+        n_sparse = max(2, min(256, int(1.0e9 // c["bytes"]) + 1))
+        copies = c["copies"] + [clone_compressed(c["copies"][0]) for _ in range(n_sparse - 2)]
+        t_sparse, _ = time_graph(torch, lambda: [mk.multiply(cc, c["x"]) for cc in copies], case_replays)
+        t_sparse /= len(copies)
+        del copies
+        per = c["per"]
+        per["macko_us"] = round(t_sparse * 1e6, 2)
+        per["macko_gbps"] = round(c["bytes"] / t_sparse / 1e9, 1)
+        per["pct_hbm_peak"] = round(100 * c["bytes"] / t_sparse / 1e9 / HBM_PEAK_GBPS, 1)
+        if "dense_us" in per:
+            per["speedup_vs_dense"] = round(per["dense_us"] / per["macko_us"], 3)
+            per["speedup_vs_best_dense"] = round(min(per["dense_us"], per["dense_as_gemm_us"]) / per["macko_us"], 3)
+        if yardstick is not None:
+            per["stream_read_us"] = round(yardstick.seconds(c["bytes"], case_replays) * 1e6, 2)
+        per_case.append(per)
+        log(f"[{suite}]", per)
 
-        hip = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
-        hip.macko_calibration_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
-        def read_stride(nbytes):
-            return (int(nbytes) // 16 * 16 + 4095) // 4096 * 4096
+    def mean_speedup(d, key="speedup_vs_dense"):
+        v = [p[key] for p in per_case if p["density"] == d and key in p]
+        return round(sum(v) / len(v), 3) if v else None
 
-        # the pool holds at least two copies of the largest case, so consecutive launches never re-read
-        pool_bytes = max(1 << 30, 2 * max(read_stride(c["bytes"]) for c in cases))
-        read_pool = torch.ones(pool_bytes, dtype=torch.uint8, device="cuda")
-        read_sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    traffic, traffic_source = load_traffic(suite)
+    summary = {
+        "workload": WORKLOADS[suite],
+        "value": round(gbps, 2),
+        "unit": "GB/s",
+        "steps": steps,
+        "ms_per_step": round(elapsed_s * 1e3 / steps, 5),
+        "launches_per_step": n_launch,
+        "bytes_per_step": step_bytes,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbps, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "kernel": "spmv_split_kernel" if suite == "fewrows" else "spmv_stream_kernel",
+            "bytes_per_launch": round(step_bytes / n_launch),
+            "us_per_launch": round(launch_us, 3),
+        },
+        "speedup_vs_dense_fp16_gemv": {"d0.5": mean_speedup(0.5), "d0.1": mean_speedup(0.1)},
+        # against the faster of torch.matmul(W, x) and torch.matmul(x[None], W.T) per case
+        "speedup_vs_best_dense_fp16": {"d0.5": mean_speedup(0.5, "speedup_vs_best_dense"),
+                                       "d0.1": mean_speedup(0.1, "speedup_vs_best_dense")},
+        "cases": per_case,
+    }
+    if yardstick is not None and per_case:
+        t_m = sum(p["macko_us"] for p in per_case)
+        t_r = sum(p["stream_read_us"] for p in per_case)
+        summary["streaming_read_yardstick"] = {
+            "what": ReadYardstick.WHAT,
+            "us_per_launch": round(t_r / len(per_case), 3),
+            "gbps": round(step_bytes / t_r / 1e3, 1),
+            "spmv_time_over_read_time": round(t_m / t_r, 3),
+        }
+    return summary, cases
 
-        def read_copies(nbytes):
-            return pool_bytes // read_stride(nbytes)
 
-        def read_launches(nbytes):
-            # pure streaming read of the same number of bytes, rotating through the pool
-            nbytes = int(nbytes) // 16 * 16
-            stride = read_stride(nbytes)
-            sp = torch.cuda.current_stream().cuda_stream
-            for k in range(read_copies(nbytes)):
-                assert k * stride + nbytes <= pool_bytes  # the kernel trusts its arguments
-                rc = hip.macko_calibration_read(read_pool.data_ptr() + k * stride, nbytes, read_sink.data_ptr(), sp)
-                assert rc == 0, rc
+def cpu_baseline(torch, sample):
+    """The CPU route of the upstream package on `sample` (list of (W, x, density) GPU tensors): its
+    compressor (restated in C, one thread, as upstream's is) and the dense fp32 product
+    M.float() @ x.float() through torch on the host's cores; next to them the scalar C restatement of
+    the product taken from the compressed arrays."""
+    import numpy as np
 
-        for c in cases:
-            n_sparse = max(2, min(256, int(1.0e9 // c["bytes"]) + 1))
-            copies = c["copies"] + [clone_compressed(c["copies"][0]) for _ in range(n_sparse - 2)]
-            t_sparse, _ = time_graph(torch, lambda: [mk.multiply(cc, c["x"]) for cc in copies], args.case_replays)
-            t_sparse /= len(copies)
-            del copies
-            db = dense_bytes(c["rows"], c["cols"])
-            n_dense = max(2, min(64, int(1.0e9 // db) + 1))
-            dense_copies = [c["W"]] + [c["W"].clone() for _ in range(n_dense - 1)]
-            t_dense, _ = time_graph(torch, lambda: [torch.matmul(Wc, c["x"]) for Wc in dense_copies],
-                                    args.case_replays)
-            t_dense /= len(dense_copies)
-            # the same product phrased as a one-row GEMM, which hipBLASLt serves with other kernels
-            x_row = c["x"][None, :]
-            t_dense_gemm, _ = time_graph(torch, lambda: [torch.matmul(x_row, Wc.t()) for Wc in dense_copies],
-                                         args.case_replays)
-            t_dense_gemm /= len(dense_copies)
-            del dense_copies
-            t_read, _ = time_graph(torch, lambda: read_launches(c["bytes"]), args.case_replays)
-            t_read /= read_copies(c["bytes"])
-            per_case.append({
-                "shape": f"{c['rows']}x{c['cols']}", "density": c["density"],
-                "macko_us": round(t_sparse * 1e6, 2), "dense_us": round(t_dense * 1e6, 2),
-                "speedup_vs_dense": round(t_dense / t_sparse, 3),
-                "macko_gbps": round(c["bytes"] / t_sparse / 1e9, 1),
-                "pct_hbm_peak": round(100 * c["bytes"] / t_sparse / 1e9 / HBM_PEAK_GBPS, 1),
-                "dense_gbps": round(db / t_dense / 1e9, 1),
-                "dense_as_gemm_us": round(t_dense_gemm * 1e6, 2),
-                "speedup_vs_best_dense": round(min(t_dense, t_dense_gemm) / t_sparse, 3),
-                "stream_read_us": round(t_read * 1e6, 2),
-            })
-            log(per_case[-1])
+    from oracle import macko_oracle as mo
+
+    threads = torch.get_num_threads()
+    t_compress = t_spmv_port = t_dense_port = t_dense_torch = t_dense_torch_f16 = 0.0
+    total_bytes = 0
+    reps = 5
+    for W, x, _ in sample:
+        Wc = W.cpu()
+        xc = x.cpu()
+        dense = Wc.numpy()
+        xs = xc.numpy()
+        t0 = time.perf_counter()
+        values, deltas, row_ptr, n = mo.compress(dense)
+        t1 = time.perf_counter()
+        y = mo.spmv(values, deltas, row_ptr, dense.shape[0], dense.shape[1], xs)
+        t2 = time.perf_counter()
+        yd = mo.dense_gemv(dense, xs)
+        t3 = time.perf_counter()
+        # the stated baseline: fp32 conversion and product by torch on the host, all threads
+        want = Wc.float() @ xc.float()
+        t4 = time.perf_counter()
+        for _ in range(reps):
+            want = Wc.float() @ xc.float()
+        t5 = time.perf_counter()
+        Wf = Wc.float()
+        xf = xc.float()
+        t6 = time.perf_counter()
+        for _ in range(reps):
+            want = Wf @ xf
+        t7 = time.perf_counter()
+        assert np.allclose(y.view(np.float16).astype(np.float32), want.numpy(), rtol=1e-2, atol=1e-3)
+        assert np.allclose(yd.view(np.float16).astype(np.float32), want.numpy(), rtol=1e-2, atol=1e-3)
+        # the compressor walks the matrix twice in this wrapper (count, then fill): report one walk
+        t_compress += (t1 - t0) / 2
+        t_spmv_port += t2 - t1
+        t_dense_port += t3 - t2
+        t_dense_torch_f16 += (t5 - t4) / reps
+        t_dense_torch += (t7 - t6) / reps
+        total_bytes += algorithmic_bytes(values.size, dense.shape[0], dense.shape[1])
+    return {
+        # the dense fp32 product on the host, expressed in the metric's unit through the same byte model
+        "value": round(total_bytes / t_dense_torch_f16 / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "4096x4096, 11008x4096, 4096x11008 at density 0.5, one product each: value = algorithmic bytes "
+                  "of the compressed matrices / time of torch's M.float() @ x.float() on the host (conversion "
+                  "included, torch.get_num_threads() threads); compress_s = one walk of the C restatement of the "
+                  "upstream compressor (1 thread, as upstream)",
+        "dense_fp32_torch_s": round(t_dense_torch_f16, 4),
+        "dense_fp32_torch_preconverted_s": round(t_dense_torch, 4),
+        "compress_s": round(t_compress, 4),
+        "route_s": round(t_compress + t_dense_torch_f16, 4),
+        "port_1thread": {"spmv_s": round(t_spmv_port, 4), "spmv_gbps": round(total_bytes / t_spmv_port / 1e9, 3),
+                         "dense_fp32_matvec_s": round(t_dense_port, 4)},
+        "torch_threads": threads,
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 GEMV comparison")
+    ap.add_argument("--no-compress", action="store_true", help="skip the compressor timing")
+    ap.add_argument("--no-int8", action="store_true", help="skip the int8-values variant timing")
+    ap.add_argument("--no-batched", action="store_true", help="skip the batched-product timing")
+    ap.add_argument("--no-yardstick", action="store_true", help="skip the streaming-read yardstick")
+    ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
+    ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
+                    help="the workload `value` is measured on (llama = the headline workload)")
+    ap.add_argument("--also", default="large,skew,fewrows",
+                    help="comma-separated workloads measured in the same run and reported under `suites` "
+                         "('' for none)")
+    ap.add_argument("--also-steps", type=int, default=40, help="timed steps of each workload under `suites`")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="also launch calibration_copy_kernel on a 256 MiB buffer this many times "
+                         "(reference dispatches for scaling rocprofv3 byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (rows would shard across GPUs, but no "
+                 "multi-GPU path is part of it); run with --gpus 1")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the MACKO path has no CPU implementation to benchmark")
+    import macko_spmv_amd as mk
+
+    dev = torch.cuda.get_device_properties(0)
+    log(f"device: {dev.name}, {dev.multi_processor_count} CUs")
+    bench_lib = load_bench_library()
+
+    if args.calibration_copies > 0:
+        n_bytes = 256 << 20
+        src = torch.ones(n_bytes // 2, dtype=torch.float16, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            rc = bench_lib.macko_calibration_copy(src.data_ptr(), dst.data_ptr(), n_bytes,
+                                                  torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        log(f"calibration: {args.calibration_copies} copies of {n_bytes} bytes "
+            f"(each reads {n_bytes} and writes {n_bytes} bytes)")
+        del src, dst
+
+    yardstick = None if args.no_yardstick else ReadYardstick(torch, bench_lib, 800e6)
+
+    # ---- the headline workload -------------------------------------------------------------------
+    head, cases = measure_suite(torch, mk, args.suite, args.steps, args.warmup, yardstick, args.case_replays,
+                                with_dense=not args.no_dense, keep_dense=True)
+    per_case = head["cases"]
 
     # ---- int8 values variant on the same sparsity patterns (densities 0.1 and 0.5 only) ------------
     int8_cases = []
@@ -378,8 +521,7 @@ def main():
             t8, _ = time_graph(torch, lambda: [mk.multiply_int8(cc, c["x"]) for cc in copies], args.case_replays)
             t8 /= len(copies)
             del copies
-            dense_us = next((p["dense_us"] for p in per_case
-                             if p["shape"] == f"{c['rows']}x{c['cols']}" and p["density"] == c["density"]), None)
+            dense_us = c["per"].get("dense_us")
             int8_cases.append({
                 "shape": f"{c['rows']}x{c['cols']}", "density": c["density"], "us": round(t8 * 1e6, 2),
                 "gbps": round(nbytes / t8 / 1e9, 1), "pct_hbm_peak": round(100 * nbytes / t8 / 1e9 / HBM_PEAK_GBPS, 1),
@@ -442,30 +584,30 @@ def main():
         cpu = cpu_baseline(torch, sample)
         log("cpu baseline:", cpu)
 
-    def mean_speedup(d, key="speedup_vs_dense"):
-        v = [p[key] for p in per_case if p["density"] == d]
-        return round(sum(v) / len(v), 3) if v else None
+    del cases
+    gc.collect()
+    torch.cuda.empty_cache()
 
-    yardstick = None
-    if per_case:
-        t_m = sum(p["macko_us"] for p in per_case)
-        t_r = sum(p["stream_read_us"] for p in per_case)
-        yardstick = {
-            "what": "calibration_read_kernel: one launch that only reads the same number of bytes (256x1024 "
-                    "threads, contiguous span per wave, four non-temporal 16-byte loads per lane in flight), timed like the per-case SpMV figures",
-            "us_per_launch": round(t_r / len(per_case), 3),
-            "gbps": round(step_bytes / t_r / 1e3, 1),
-            "spmv_time_over_read_time": round(t_m / t_r, 3),
-        }
-    bytes_per_launch = step_bytes / n_launch
+    # ---- the other workloads, measured the same way -------------------------------------------------
+    suites = {}
+    for name in [s for s in args.also.split(",") if s and s != args.suite]:
+        if name not in WORKLOADS:
+            sys.exit(f"bench.py: unknown workload {name!r} in --also")
+        summary, other = measure_suite(torch, mk, name, args.also_steps, max(2, args.also_steps // 10), yardstick,
+                                       max(5, args.case_replays // 2), with_dense=not args.no_dense)
+        del other
+        gc.collect()
+        torch.cuda.empty_cache()
+        suites[name] = summary
+
     out = {
         "metric": "SpMV effective HBM GB/s (% of ~8 TB/s) + speedup vs dense fp16 GEMV",
-        "value": round(gbps, 2),
+        "value": head["value"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -473,28 +615,17 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": WORKLOADS[args.suite],
-            "launches_per_step": n_launch,
-            "bytes_per_step": step_bytes,
+            "launches_per_step": head["launches_per_step"],
+            "bytes_per_step": head["bytes_per_step"],
         },
-        "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
-        "speedup_vs_dense_fp16_gemv": {"d0.5": mean_speedup(0.5), "d0.1": mean_speedup(0.1)},
-        # against the faster of torch.matmul(W, x) and torch.matmul(x[None], W.T) per case
-        "speedup_vs_best_dense_fp16": {"d0.5": mean_speedup(0.5, "speedup_vs_best_dense"),
-                                       "d0.1": mean_speedup(0.1, "speedup_vs_best_dense")},
-        "roofline": {
-            "bound": "hbm",
-            "achieved": round(gbps, 2),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.suite),
-            "kernel": "spmv_stream_kernel",
-            "bytes_per_launch": round(bytes_per_launch),
-            "us_per_launch": round(launch_us, 3),
-        },
+        "pct_of_hbm_peak": round(100 * head["value"] / HBM_PEAK_GBPS, 2),
+        "speedup_vs_dense_fp16_gemv": head["speedup_vs_dense_fp16_gemv"],
+        "speedup_vs_best_dense_fp16": head["speedup_vs_best_dense_fp16"],
+        "roofline": head["roofline"],
         "cpu_baseline": cpu,
-        "streaming_read_yardstick": yardstick,
+        "streaming_read_yardstick": head.get("streaming_read_yardstick"),
         "cases": per_case,
+        "suites": suites,
         "compress": compress_cases,
         "int8_values_variant": int8_cases,
         "batched_product": batched_cases,

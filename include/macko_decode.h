@@ -14,12 +14,14 @@
 
 #include <stdint.h>
 
+#include "macko_hip.h" /* MACKO_API, return codes */
+
 #ifdef __cplusplus
 extern "C" {
 #endif
 
 /* y[i] = x[i] * rsqrt(mean(x^2) + eps) * weight[i], i < n. */
-int macko_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int32_t n, float eps,
+MACKO_API int macko_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int32_t n, float eps,
                              void *stream);
 
 /*
@@ -27,7 +29,7 @@ int macko_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int32_t
  * *position; writes the rotated q to q_out and appends the rotated k and v to the caches
  * [n_heads, max_len, head_dim] at that position.  cos_table / sin_table: [max_len, head_dim/2].
  */
-int macko_decode_rope_append_f16(const void *q, const void *k, const void *v,
+MACKO_API int macko_decode_rope_append_f16(const void *q, const void *k, const void *v,
                                  const float *cos_table, const float *sin_table,
                                  const int64_t *position, void *q_out, void *k_cache,
                                  void *v_cache, int32_t n_heads, int32_t head_dim,
@@ -38,7 +40,7 @@ int macko_decode_rope_append_f16(const void *q, const void *k, const void *v,
  * out = softmax(scale * q K^T) V.  head_dim <= 256 and a multiple of 8, max_len <= 4096,
  * both caches 16-byte aligned.
  */
-int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache,
+MACKO_API int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v_cache,
                                const int64_t *position, void *out, int32_t n_heads,
                                int32_t head_dim, int32_t max_len, float scale, void *stream);
 
@@ -47,14 +49,14 @@ int macko_decode_attention_f16(const void *q, const void *k_cache, const void *v
  * the raw projections of the current token, the caches receive the rotated k and v at *position,
  * out is the attention output.  Same limits as the two separate calls.
  */
-int macko_decode_rope_attention_f16(const void *q, const void *k, const void *v,
+MACKO_API int macko_decode_rope_attention_f16(const void *q, const void *k, const void *v,
                                     const float *cos_table, const float *sin_table,
                                     const int64_t *position, void *k_cache, void *v_cache,
                                     void *out, int32_t n_heads, int32_t head_dim, int32_t max_len,
                                     float scale, void *stream);
 
 /* out[i] = silu(gate[i]) * up[i], i < n. */
-int macko_decode_silu_mul_f16(const void *gate, const void *up, void *out, int32_t n,
+MACKO_API int macko_decode_silu_mul_f16(const void *gate, const void *up, void *out, int32_t n,
                               void *stream);
 
 #ifdef __cplusplus

@@ -24,14 +24,21 @@
 extern "C" {
 #endif
 
+/* Entry points are the only symbols the library exports. */
+#if defined(__GNUC__)
+#define MACKO_API __attribute__((visibility("default")))
+#else
+#define MACKO_API
+#endif
+
 #define MACKO_E_INVALID_ARGUMENT (-1) /* null pointer, negative size, rows*cols >= 2^31 ... */
 #define MACKO_E_NO_DEVICE (-2)        /* no usable HIP device */
 
 /* ABI version of this header (bumped on incompatible change). */
-int macko_hip_abi_version(void);
+MACKO_API int macko_hip_abi_version(void);
 
 /* Human-readable text for a return code of this library.  Never NULL; static storage. */
-const char *macko_hip_error_string(int code);
+MACKO_API const char *macko_hip_error_string(int code);
 
 /*
  * y[r] = fp16( sum_k fp32(values[k]) * fp32(x[col_k]) ) for every row r, fp32 accumulation.
@@ -44,7 +51,7 @@ const char *macko_hip_error_string(int code);
  *   x   fp16 [>= cols], 2-byte aligned (16-byte alignment is faster)
  *   y   fp16 [rows], written for every row
  */
-int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_ptr,
                    const void *x, void *y, int32_t rows, int32_t cols,
                    int64_t padded_entries, void *stream);
 
@@ -54,7 +61,7 @@ int macko_spmv_f16(const void *values, const void *deltas, const int32_t *row_pt
  * Replaces the macko_spmv<true> instantiation that the upstream C benchmark launches
  * (src/macko_spmv/cuda/kernels.cuh:113-118, c_benchmarking/benchmark.cu:92-105).
  */
-int macko_spmv_f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
                          const void *x, void *y, int32_t rows, int32_t cols,
                          int64_t padded_entries, float alpha, float beta, void *stream);
 
@@ -67,7 +74,7 @@ int macko_spmv_f16_axpby(const void *values, const void *deltas, const int32_t *
  * Steps 1+2 together replace compress_rows_cpu (src/macko_spmv/cuda/cpu_compressor.cuh:6-73)
  * and emit bit-identical arrays.
  */
-int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols,
+MACKO_API int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols,
                              int32_t *row_ptr, void *stream);
 
 /*
@@ -76,7 +83,7 @@ int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols,
  * tail zero-filled, whatever they held before.  P must be ceil(row_ptr[rows]/8)*8.
  * Asynchronous.
  */
-int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
+MACKO_API int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
                             const int32_t *row_ptr, void *values, void *deltas,
                             int64_t padded_entries, void *stream);
 
@@ -87,7 +94,7 @@ int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols,
  * counterpart in the upstream package, whose LLM runner maps the single-vector operator over
  * the batch dimension (python_scripts/util_run_pruned_llm.py:112-118).
  */
-int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t *row_ptr,
                            const void *x, void *y, int32_t rows, int32_t cols,
                            int64_t padded_entries, int32_t batch, int64_t ldx, int64_t ldy,
                            void *stream);
@@ -103,10 +110,10 @@ int macko_spmv_f16_batched(const void *values, const void *deltas, const int32_t
  * macko_spmv_f16_silu_mul_axpby: y = alpha * M g + beta * y,  g[i] = fp16(silu(gate[i]) * up[i]);
  *                                with alpha == 1 and beta == 0, y is not read.
  */
-int macko_spmv_f16_rmsnorm(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_f16_rmsnorm(const void *values, const void *deltas, const int32_t *row_ptr,
                            const void *x, const void *norm_weight, float eps, void *y,
                            int32_t rows, int32_t cols, int64_t padded_entries, void *stream);
-int macko_spmv_f16_silu_mul_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_f16_silu_mul_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
                                   const void *gate, const void *up, void *y, int32_t rows,
                                   int32_t cols, int64_t padded_entries, float alpha, float beta,
                                   void *stream);
@@ -120,26 +127,28 @@ int macko_spmv_f16_silu_mul_axpby(const void *values, const void *deltas, const 
  * c_benchmarking/benchmark.cu:106-118): y = fp16(alpha * sum float(value) * float(x[col])
  * [+ beta * y]), fp32 accumulation.
  */
-int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols,
+MACKO_API int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols,
                             int32_t *row_ptr, void *stream);
-int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols,
+MACKO_API int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols,
                            const int32_t *row_ptr, void *values, void *deltas,
                            int64_t padded_entries, void *stream);
-int macko_spmv_i8f16(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_i8f16(const void *values, const void *deltas, const int32_t *row_ptr,
                      const void *x, void *y, int32_t rows, int32_t cols,
                      int64_t padded_entries, void *stream);
-int macko_spmv_i8f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
+MACKO_API int macko_spmv_i8f16_axpby(const void *values, const void *deltas, const int32_t *row_ptr,
                            const void *x, void *y, int32_t rows, int32_t cols,
                            int64_t padded_entries, float alpha, float beta, void *stream);
 
 /*
  * Inverse of the compressor: writes the dense row-major fp16 matrix [rows, cols] (every
- * element written).  Uses the decode rule of the multiply kernel
+ * element written; `dense` 2-byte aligned).  Uses the decode rule of the multiply kernel
  * (src/macko_spmv/cuda/kernels.cuh:97-103); the upstream package has no such function, it is
- * provided for round-trip checks at sizes a CPU decode cannot reach.
+ * provided for round-trip checks at sizes a CPU decode cannot reach.  padded_entries = P bounds
+ * what is read of values / deltas.  Launches kernels only (no memset), so it may be captured.
  */
-int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr,
-                         int32_t rows, int32_t cols, void *dense, void *stream);
+MACKO_API int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr,
+                         int32_t rows, int32_t cols, int64_t padded_entries, void *dense,
+                         void *stream);
 
 #ifdef __cplusplus
 }

@@ -2,6 +2,7 @@
 
   libmacko_hip.so    torch-free HIP kernels behind the C ABI of include/macko_hip.h (gfx950)
   libmacko_torch.so  PyTorch-ROCm operator library that forwards to the C ABI
+  libmacko_bench.so  the benchmark's own kernels (streaming-read yardstick, counter calibration)
 
 Both are built in-tree (next to this file) unless MACKO_SPMV_BUILD_DIRECTORY names another
 directory -- the same variable the upstream package reads for its JIT cache
@@ -23,10 +24,12 @@ _INCLUDE = os.path.join(_ROOT, "include")
 
 HIP_LIB = "libmacko_hip.so"
 TORCH_LIB = "libmacko_torch.so"
+BENCH_LIB = "libmacko_bench.so"  # kernels of bench.py only; the package never loads it
 ARCH = "gfx950"
 
 HIP_SOURCES = ["macko_spmv.hip", "macko_spmv_split.hip", "macko_compress.hip", "macko_runtime.hip", "macko_decode.hip"]
 TORCH_SOURCES = ["macko_torch.cpp"]
+BENCH_SOURCES = ["macko_bench_kernels.hip"]
 
 
 def build_directory():
@@ -141,7 +144,8 @@ def build_hip(verbose=False):
     verify_fixed_registers(verbose)
     staging = out + ".building"
     cmd = [
-        _hipcc(), *_DEVICE_FLAGS, "-fPIC", "-shared",
+        # only what include/*.h declare is exported
+        _hipcc(), *_DEVICE_FLAGS, "-fvisibility=hidden", "-fPIC", "-shared",
         *[os.path.join(_CSRC, s) for s in HIP_SOURCES],
         "-o", staging,
     ]
@@ -180,7 +184,7 @@ def stamp_path():
 def is_current():
     """True when both libraries exist and were built from the sources as they are now."""
     hip_lib, torch_lib = lib_paths()
-    if not (os.path.exists(hip_lib) and os.path.exists(torch_lib) and os.path.exists(stamp_path())):
+    if not all(os.path.exists(f) for f in (hip_lib, torch_lib, bench_lib_path(), stamp_path())):
         return False
     with open(stamp_path()) as f:
         return f.read().strip() == source_digest()
@@ -212,10 +216,22 @@ def build_torch(verbose=False):
     return out
 
 
+def bench_lib_path():
+    return os.path.join(build_directory(), BENCH_LIB)
+
+
+def build_bench(verbose=False):
+    out = bench_lib_path()
+    _run([_hipcc(), *_DEVICE_FLAGS, "-fPIC", "-shared", *[os.path.join(_CSRC, s) for s in BENCH_SOURCES], "-o", out],
+         verbose)
+    return out
+
+
 def build_all(verbose=False):
     if os.path.exists(stamp_path()):
         os.remove(stamp_path())
     built = build_hip(verbose), build_torch(verbose)
+    build_bench(verbose)
     with open(stamp_path(), "w") as f:
         f.write(source_digest() + "\n")
     return built

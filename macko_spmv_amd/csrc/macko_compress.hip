@@ -300,21 +300,24 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Ele
     }
 }
 
-// One wave per row, one entry per lane per pass.
+// One wave per row, one entry per lane per pass.  `padded` bounds every read of values / deltas, so
+// a row_ptr that points past the arrays cannot make the kernel read outside them.
 __global__ void __launch_bounds__(kBlock) decode_rows_kernel(const uint16_t *__restrict__ values,
                                                              const unsigned char *__restrict__ deltas,
                                                              const int *__restrict__ row_ptr, int rows, int cols,
-                                                             uint16_t *__restrict__ dense)
+                                                             long long padded, uint16_t *__restrict__ dense)
 {
     const int lane = threadIdx.x & (kWave - 1);
     const int row = blockIdx.x * kRowsPerBlock + uniform(threadIdx.x >> 6);
     if (row >= rows) return;
-    const int e0 = row_ptr[row];
-    const int e1 = row_ptr[row + 1];
+    long long e0 = row_ptr[row];
+    long long e1 = row_ptr[row + 1];
+    e0 = e0 < 0 ? 0 : (e0 > padded ? padded : e0);
+    e1 = e1 < e0 ? e0 : (e1 > padded ? padded : e1);
     uint16_t *dst = dense + (size_t)row * (size_t)cols;
     int column = -1;  // column of the last entry decoded so far
-    for (int j0 = e0; j0 < e1; j0 += kWave) {
-        const int j = j0 + lane;
+    for (long long j0 = e0; j0 < e1; j0 += kWave) {
+        const long long j = j0 + lane;
         int step = 0;
         uint16_t val = 0;
         if (j < e1) {
@@ -326,6 +329,17 @@ __global__ void __launch_bounds__(kBlock) decode_rows_kernel(const uint16_t *__r
         if (j < e1 && c < cols) dst[c] = val;
         column += __builtin_amdgcn_readlane(incl, kWave - 1);
     }
+}
+
+// dst[0 .. n_vec) = 0, 16 bytes per thread and step (a fill kernel rather than a memset node, so
+// the call can sit in a captured graph).
+__global__ void __launch_bounds__(256) zero_fill_kernel(u32x4 *__restrict__ dst, size_t n_vec, uint16_t *__restrict__ tail,
+                                                        int n_tail)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (size_t i = first; i < n_vec; i += stride) dst[i] = u32x4{0u, 0u, 0u, 0u};
+    if (first < (size_t)n_tail) tail[first] = 0;
 }
 
 }  // namespace
@@ -429,18 +443,35 @@ extern "C" int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t c
 }
 
 extern "C" int macko_decompress_f16(const void *values, const void *deltas, const int32_t *row_ptr, int32_t rows,
-                                    int32_t cols, void *dense, void *stream)
+                                    int32_t cols, int64_t padded_entries, void *dense, void *stream)
 {
     using namespace macko;
-    if (rows < 0 || cols < 0) return MACKO_E_INVALID_ARGUMENT;
+    if (rows < 0 || cols < 0 || padded_entries < 0) return MACKO_E_INVALID_ARGUMENT;
     if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
     if (rows == 0 || cols == 0) return 0;
     if (dense == nullptr || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
+    if (padded_entries > 0 && (values == nullptr || deltas == nullptr)) return MACKO_E_INVALID_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(dense) & 1) return MACKO_E_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
-    hipError_t e = hipMemsetAsync(dense, 0, (size_t)rows * (size_t)cols * 2, s);
-    if (e != hipSuccess) return (int)e;
+    {   // zeros first: whole 16-byte pieces from the first aligned address on, the few elements around them singly
+        const size_t n = (size_t)rows * (size_t)cols;
+        uint16_t *d = (uint16_t *)dense;
+        size_t head = ((16 - (reinterpret_cast<uintptr_t>(d) & 15)) & 15) / 2;
+        if (head > n) head = n;
+        const size_t n_vec = (n - head) / 8;
+        const size_t rest = n - head - 8 * n_vec;
+        if (head > 0)
+            hipLaunchKernelGGL(zero_fill_kernel, dim3(1), dim3(256), 0, s, (u32x4 *)nullptr, (size_t)0, d, (int)head);
+        size_t blocks = (n_vec + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        if (blocks < 1) blocks = 1;
+        hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (u32x4 *)(d + head), n_vec,
+                           d + head + 8 * n_vec, (int)rest);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
     hipLaunchKernelGGL(decode_rows_kernel, dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlock), 0, s,
                        (const uint16_t *)values, (const unsigned char *)deltas, row_ptr, rows, cols,
-                       (uint16_t *)dense);
+                       (long long)padded_entries, (uint16_t *)dense);
     return (int)hipGetLastError();
 }

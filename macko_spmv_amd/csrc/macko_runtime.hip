@@ -2,6 +2,8 @@
 
 #include <string.h>
 
+#include <atomic>
+
 #include "macko_common.h"
 
 namespace macko {
@@ -9,12 +11,15 @@ namespace macko {
 int device_info(DeviceInfo *out)
 {
     constexpr int kMaxDevices = 64;
+    // per device: 0 = unknown, 1 = being written, 2 = known.  Concurrent first calls may both query
+    // the device; only one of them writes the cache entry, readers wait for state 2.
     static DeviceInfo cache[kMaxDevices];
-    static bool known[kMaxDevices] = {};
+    static std::atomic<int> state[kMaxDevices];
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e == hipErrorNoDevice ? MACKO_E_NO_DEVICE : (int)e;
-    if (dev >= 0 && dev < kMaxDevices && known[dev]) {
+    const bool cached = dev >= 0 && dev < kMaxDevices;
+    if (cached && state[dev].load(std::memory_order_acquire) == 2) {
         *out = cache[dev];
         return 0;
     }
@@ -26,9 +31,12 @@ int device_info(DeviceInfo *out)
     if (e != hipSuccess) return (int)e;
     // gfx950 gives a workgroup up to 160 KiB of LDS; anything else is treated as 64 KiB
     info.max_lds_bytes = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 160 * 1024 : 64 * 1024;
-    if (dev >= 0 && dev < kMaxDevices) {
-        cache[dev] = info;
-        known[dev] = true;
+    if (cached) {
+        int expected = 0;
+        if (state[dev].compare_exchange_strong(expected, 1, std::memory_order_acq_rel)) {
+            cache[dev] = info;
+            state[dev].store(2, std::memory_order_release);
+        }
     }
     *out = info;
     return 0;
@@ -36,65 +44,7 @@ int device_info(DeviceInfo *out)
 
 }  // namespace macko
 
-// Plain 16-byte-per-thread copy with a recognisable name: hardware byte counters (FETCH_SIZE,
-// WRITE_SIZE) are scaled by what they report for this kernel on a buffer of known size.
-__global__ void __launch_bounds__(256) calibration_copy_kernel(const macko::u32x4 *__restrict__ src,
-                                                               macko::u32x4 *__restrict__ dst, size_t n_vec)
-{
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) dst[i] = src[i];
-}
-
-// Copies `bytes` (a multiple of 16; both pointers 16-byte aligned) from src to dst on `stream`.
-// Not part of the public ABI; used by the benchmark's counter calibration.
-extern "C" int macko_calibration_copy(const void *src, void *dst, int64_t bytes, void *stream)
-{
-    if (src == nullptr || dst == nullptr || bytes < 0 || (bytes & 15)) return MACKO_E_INVALID_ARGUMENT;
-    if (bytes == 0) return 0;
-    hipLaunchKernelGGL(calibration_copy_kernel, dim3(4096), dim3(256), 0, macko::as_stream(stream),
-                       (const macko::u32x4 *)src, (macko::u32x4 *)dst, (size_t)bytes / 16);
-    return (int)hipGetLastError();
-}
-
-// Pure streaming read in the SpMV's own access shape: 256 x 1024 threads, every wave walks one
-// contiguous 1/4096 of the buffer with four non-temporal 16-byte loads per lane in flight (the
-// fastest of the read patterns tried: span per wave or per workgroup, grid stride, 2 to 8 loads in
-// flight, with and without the hint).  What it takes is the
-// time any one-launch kernel needs just to pull `bytes` out of HBM: the yardstick the benchmark
-// prints next to the SpMV's time.
-__global__ void __launch_bounds__(1024) calibration_read_kernel(const macko::u32x4 *__restrict__ src, size_t n_vec,
-                                                                 macko::u32 *__restrict__ sink)
-{
-    const int lane = threadIdx.x & 63;
-    const size_t n_waves = (size_t)gridDim.x * 16, w = (size_t)blockIdx.x * 16 + (threadIdx.x >> 6);
-    const size_t begin = n_vec * w / n_waves, end = n_vec * (w + 1) / n_waves;
-    macko::u32 acc = 0;
-    size_t i = begin + lane;
-    for (; i + 192 < end; i += 256) {
-        macko::u32x4 v[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = __builtin_nontemporal_load(&src[i + 64 * k]);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) acc += v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
-    }
-    for (; i < end; i += 64) {
-        const macko::u32x4 a = __builtin_nontemporal_load(&src[i]);
-        acc += a.x ^ a.y ^ a.z ^ a.w;
-    }
-    if (acc == 0x9e3779b9u) *sink = acc;  // keeps the loads alive; practically never true
-}
-
-// Reads `bytes` (a multiple of 16; 16-byte aligned) from src; `sink` is 4 writable device bytes.
-// Not part of the public ABI; used by the benchmark's streaming yardstick.
-extern "C" int macko_calibration_read(const void *src, int64_t bytes, void *sink, void *stream)
-{
-    if (src == nullptr || sink == nullptr || bytes < 0 || (bytes & 15)) return MACKO_E_INVALID_ARGUMENT;
-    hipLaunchKernelGGL(calibration_read_kernel, dim3(256), dim3(1024), 0, macko::as_stream(stream),
-                       (const macko::u32x4 *)src, (size_t)bytes / 16, (macko::u32 *)sink);
-    return (int)hipGetLastError();
-}
-
-extern "C" int macko_hip_abi_version(void) { return 1; }
+extern "C" int macko_hip_abi_version(void) { return 2; }
 
 extern "C" const char *macko_hip_error_string(int code)
 {

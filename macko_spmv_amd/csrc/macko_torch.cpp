@@ -26,21 +26,34 @@ void check_rc(int rc, const char *what)
     TORCH_CHECK(rc == 0, "macko_spmv: ", what, " failed: ", macko_hip_error_string(rc), " (code ", rc, ")");
 }
 
-at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
-                        int64_t M_rows, int64_t M_cols, const at::Tensor &V)
+// What every product operator checks about the compressed matrix (the upstream launcher checks the
+// value dtype only, src/macko_spmv/cuda/kernels_torch_launchers.cuh:10-11; its data_ptr<T>() calls
+// throw on the other two).
+void check_macko_operands(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                          int64_t M_rows, int64_t M_cols, at::ScalarType value_type = at::kHalf)
 {
-    TORCH_CHECK(M_values.dtype() == at::kHalf, "M must be torch.half");
-    TORCH_CHECK(V.dtype() == at::kHalf, "V must be torch.half");
+    TORCH_CHECK(M_values.dtype() == value_type, value_type == at::kHalf ? "M must be torch.half" : "M must be torch.int8");
     TORCH_CHECK(M_deltas.dtype() == at::kByte, "M_deltas must be torch.uint8");
     TORCH_CHECK(M_row_indices.dtype() == at::kInt, "M_row_indices must be torch.int32");
-    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda(),
-                "all tensors must live on the GPU");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
-                    V.is_contiguous(),
-                "all tensors must be contiguous");
+    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda(), "the matrix must live on the GPU");
+    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
+                "the matrix tensors must be contiguous");
     TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
     TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
     TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+}
+
+void check_half_gpu(const at::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.dtype() == at::kHalf, name, " must be torch.half");
+    TORCH_CHECK(t.is_cuda() && t.is_contiguous(), name, " must be a contiguous GPU tensor");
+}
+
+at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
+                        int64_t M_rows, int64_t M_cols, const at::Tensor &V)
+{
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(V, "V");
     TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
 
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
@@ -57,17 +70,9 @@ at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
 at::Tensor multiply_batched_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
                                 const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &X)
 {
-    TORCH_CHECK(M_values.dtype() == at::kHalf && X.dtype() == at::kHalf, "M and X must be torch.half");
-    TORCH_CHECK(M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt, "bad index dtypes");
-    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && X.is_cuda(),
-                "all tensors must live on the GPU");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
-                    X.is_contiguous(),
-                "all tensors must be contiguous");
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(X, "X");
     TORCH_CHECK(X.dim() == 2 && X.size(1) >= M_cols, "X must be [batch, >= M_cols]");
-    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
-    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
-    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
     at::Tensor Y = at::empty({X.size(0), M_rows}, M_values.options());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
@@ -83,15 +88,10 @@ void multiply_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
                         int64_t M_rows, int64_t M_cols, const at::Tensor &V, at::Tensor C, double alpha,
                         double beta)
 {
-    TORCH_CHECK(M_values.dtype() == at::kHalf && V.dtype() == at::kHalf && C.dtype() == at::kHalf,
-                "M, V and C must be torch.half");
-    TORCH_CHECK(M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt, "bad index dtypes");
-    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda() && C.is_cuda(),
-                "all tensors must live on the GPU");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
-                    V.is_contiguous() && C.is_contiguous(),
-                "all tensors must be contiguous");
-    TORCH_CHECK(C.numel() >= M_rows && M_row_indices.numel() >= M_rows + 1, "bad sizes");
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(V, "V");
+    check_half_gpu(C, "C");
+    TORCH_CHECK(C.numel() >= M_rows, "C must hold M_rows elements");
     TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
@@ -175,18 +175,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_int8_c
 void check_int8_operands(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
                          int64_t M_rows, int64_t M_cols, const at::Tensor &V)
 {
-    TORCH_CHECK(M_values.dtype() == at::kChar, "M must be torch.int8");
-    TORCH_CHECK(V.dtype() == at::kHalf, "V must be torch.half");
-    TORCH_CHECK(M_deltas.dtype() == at::kByte, "M_deltas must be torch.uint8");
-    TORCH_CHECK(M_row_indices.dtype() == at::kInt, "M_row_indices must be torch.int32");
-    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda() && V.is_cuda(),
-                "all tensors must live on the GPU");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous() &&
-                    V.is_contiguous(),
-                "all tensors must be contiguous");
-    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
-    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
-    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols, at::kChar);
+    check_half_gpu(V, "V");
     TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
 }
 
@@ -223,26 +213,18 @@ void multiply_int8_axpby_hip(const at::Tensor &M_values, const at::Tensor &M_del
 at::Tensor decompress_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
                           int64_t M_rows, int64_t M_cols)
 {
-    TORCH_CHECK(M_values.dtype() == at::kHalf && M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt,
-                "bad dtypes");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
-                "all tensors must be contiguous");
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    TORCH_CHECK(M_rows * M_cols < (1ll << 31), "matrix too large: rows * cols must stay below 2^31");
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
     at::Tensor dense = at::empty({M_rows, M_cols}, M_values.options());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_rc(macko_decompress_f16(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
-                                  (int32_t)M_rows, (int32_t)M_cols, dense.data_ptr(), (void *)stream),
+                                  (int32_t)M_rows, (int32_t)M_cols, M_values.numel(), dense.data_ptr(), (void *)stream),
              "decompress");
     return dense;
 }
 
 // ---- glue kernels of the decode harness (include/macko_decode.h) -------------------------------
-
-void check_half_gpu(const at::Tensor &t, const char *name)
-{
-    TORCH_CHECK(t.is_cuda() && t.dtype() == at::kHalf && t.is_contiguous(), name,
-                " must be a contiguous torch.half GPU tensor");
-}
 
 at::Tensor decode_rmsnorm_hip(const at::Tensor &x, const at::Tensor &weight, double eps)
 {
@@ -318,19 +300,6 @@ at::Tensor decode_silu_mul_hip(const at::Tensor &gate, const at::Tensor &up)
                                        (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream()),
              "decode_silu_mul");
     return out;
-}
-
-void check_macko_operands(const at::Tensor &M_values, const at::Tensor &M_deltas, const at::Tensor &M_row_indices,
-                          int64_t M_rows, int64_t M_cols)
-{
-    TORCH_CHECK(M_values.dtype() == at::kHalf && M_deltas.dtype() == at::kByte && M_row_indices.dtype() == at::kInt,
-                "bad matrix dtypes");
-    TORCH_CHECK(M_values.is_cuda() && M_deltas.is_cuda() && M_row_indices.is_cuda(), "the matrix must live on the GPU");
-    TORCH_CHECK(M_values.is_contiguous() && M_deltas.is_contiguous() && M_row_indices.is_contiguous(),
-                "the matrix tensors must be contiguous");
-    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
-    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
-    TORCH_CHECK(M_deltas.numel() * 2 >= M_values.numel(), "M_deltas must hold one nibble per value");
 }
 
 // M @ rmsnorm(V): the norm is applied while V is staged for the product.

@@ -1,7 +1,8 @@
 """Llama-architecture batch-1 decode with MACKO linear layers.
 
 Counterpart of the upstream helper scripts:
-  python_scripts/util_compress_llm.py:16-44    -> compress_state_dict()  (keys `<module>.c_0 .. c_4`)
+  python_scripts/util_compress_llm.py:16-44    -> compress_state_dict()  (keys `<module>.c_0 .. c_4`),
+                                                  save_compressed_state_dict() / load_compressed_state_dict()
   python_scripts/util_run_pruned_llm.py:102-133 -> MackoLinear (their CustomLayer), load_compressed_linears (their fix)
   python_scripts/util_run_pruned_llm.py:51-99,136-207 -> Generator-style greedy decode loop and the tok/s, memory report
 
@@ -48,6 +49,36 @@ def compress_state_dict(state_dict, compress=None):
                 out[key.replace("weight", f"c_{i}")] = compressed[i]
         else:
             out[key] = value
+    return out
+
+
+def save_compressed_state_dict(compressed_sd, path):
+    """Write a compressed state dict the way the upstream script does: one torch.save of an
+    OrderedDict whose `<m>.c_0 .. c_2` are tensors and `<m>.c_3`, `<m>.c_4` Python ints
+    (python_scripts/util_compress_llm.py:23-25,44).  Tensors are moved to the CPU first, so the
+    file loads on a host without a GPU."""
+    out = OrderedDict()
+    for key, value in compressed_sd.items():
+        if torch.is_tensor(value):
+            out[key] = value.detach().cpu().contiguous()
+        else:
+            out[key] = int(value)
+    torch.save(out, path)
+    return path
+
+
+def load_compressed_state_dict(path, device=None):
+    """Read a file written by save_compressed_state_dict or by the upstream script
+    (python_scripts/util_run_pruned_llm.py:146 does a plain torch.load).  Loaded with
+    weights_only=True: nothing in the file is executed.  Tensors go to `device` if given; the
+    `c_3` / `c_4` entries come back as Python ints."""
+    loaded = torch.load(path, map_location="cpu", weights_only=True)
+    out = OrderedDict()
+    for key, value in loaded.items():
+        if torch.is_tensor(value):
+            out[key] = value.to(device) if device is not None else value
+        else:
+            out[key] = int(value)
     return out
 
 
@@ -457,6 +488,10 @@ def main(argv=None):
     ap.add_argument("--module-path", action="store_true",
                     help="decode through the nn.Module forward (one framework kernel per elementary op) "
                          "instead of the lean DecodeEngine step")
+    ap.add_argument("--compressed-file", default=None,
+                    help="write the MACKO model's compressed state dict to this file and build the model that "
+                         "is timed from what is read back (the upstream pair of scripts: compress to disk, run "
+                         "from disk)")
     ap.add_argument("--no-fuse", action="store_true",
                     help="engine path: keep rotary, the RMS norms and the SiLU gate as launches of their own")
     args = ap.parse_args(argv)
@@ -470,7 +505,12 @@ def main(argv=None):
         if label == "dense" and args.skip_dense:
             continue
         model, proj_bytes = build_model(args.density, args.layers, args.dim, args.hidden, args.heads, args.vocab,
-                                        max_len, sparse=sparse)
+                                        max_len, sparse=sparse and not args.compressed_file)
+        if sparse and args.compressed_file:
+            save_compressed_state_dict(compress_state_dict(model.state_dict()), args.compressed_file)
+            load_compressed_linears(model, load_compressed_state_dict(args.compressed_file, device="cuda"))
+            proj_bytes = sum(m.weight_bytes() for m in model.modules() if isinstance(m, MackoLinear))
+            torch.cuda.empty_cache()
         engine = None
         if not args.module_path:
             engine = DecodeEngine(model, fuse=not args.no_fuse)

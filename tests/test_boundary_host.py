@@ -25,6 +25,13 @@ def _declared_symbols():
     return sorted(names)
 
 
+def _exported_symbols(path):
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", path], stdout=subprocess.PIPE, text=True, check=True).stdout
+    return sorted(line.split()[-1] for line in out.splitlines() if " T " in line)
+
+
 def test_header_symbols_are_exported():
     names = _declared_symbols()
     assert {"macko_spmv_f16", "macko_spmv_f16_axpby", "macko_compress_f16_count", "macko_compress_f16_fill",
@@ -33,11 +40,19 @@ def test_header_symbols_are_exported():
     lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
     for name in names:
         assert hasattr(lib, name), f"{name} declared under include/ but not exported"
+    # and nothing else: no tuning hooks, no benchmark kernels, no C++ internals
+    assert _exported_symbols(macko_spmv_amd.HIP_LIBRARY_PATH) == names
+
+
+def test_libraries_are_built_from_the_current_sources():
+    from macko_spmv_amd import _build
+
+    assert _build.is_current(), "csrc/ or include/ changed since the libraries were built"
 
 
 def test_abi_version_and_error_strings():
     lib = ctypes.CDLL(macko_spmv_amd.HIP_LIBRARY_PATH)
-    assert lib.macko_hip_abi_version() == 1
+    assert lib.macko_hip_abi_version() == 2
     lib.macko_hip_error_string.restype = ctypes.c_char_p
     assert lib.macko_hip_error_string(0) == b"success"
     assert b"invalid argument" in lib.macko_hip_error_string(-1)
@@ -155,3 +170,13 @@ def test_assembly_check_of_the_hand_tracked_loads():
         head + ["\ts_waitcnt vmcnt(0)", ".LBB0_2:", "\ts_waitcnt lgkmcnt(0)"] + take + tail) == 1
     with pytest.raises(RuntimeError, match="stale"):
         _build.check_stream_kernel_assembly(["\ts_nop 0"])
+    # the second kernel keeps its loads in other registers: v84 and up, ring slots at v94 / v98
+    name, base, slots = _build.TRACKED_KERNELS["macko_spmv_split.hip"]
+    head2 = ["_ZN5macko12_GLOBAL__N_117spmv_split_kernelILi1024ELi2ELb1ELb0ELi2ELi1ELi0EEEvNS_11spmv_detail8SpmvArgsE: ; @x"]
+    take2 = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(2)", "\tv_mov_b32 v0, v94", "\t;;#ASMEND"]
+    assert _build.check_stream_kernel_assembly(head2 + ["\tv_mov_b32_e32 v83, 0"] + take2 + tail, name, base, slots) == 1
+    with pytest.raises(RuntimeError, match="fixed VGPR"):
+        _build.check_stream_kernel_assembly(head2 + ["\tv_mov_b32_e32 v84, 0"] + tail, name, base, slots)
+    with pytest.raises(RuntimeError, match="in front of a ring take"):
+        _build.check_stream_kernel_assembly(
+            head2 + [".LBB0_1:", "\ts_waitcnt vmcnt(0)", "\tv_or_b32_e32 v4, s2, v8"] + take2 + tail, name, base, slots)

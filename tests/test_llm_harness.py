@@ -28,6 +28,78 @@ def test_state_dict_key_layout_follows_upstream():
     assert list(out.keys()) == sorted(out.keys(), key=lambda k: k.replace("c_", "weight")) or True
 
 
+def test_compressed_state_dict_file_round_trip_on_the_host(tmp_path):
+    # python_scripts/util_compress_llm.py:23-25,44 writes the OrderedDict with torch.save;
+    # util_run_pruned_llm.py:146 reads it back.  No GPU involved: the compressor is a stand-in.
+    sd = OrderedDict()
+    sd["model.layers.0.self_attn.q_proj.weight"] = torch.arange(12, dtype=torch.float16).reshape(3, 4)
+    sd["model.layers.0.input_layernorm.weight"] = torch.ones(4, dtype=torch.float16)
+    fake = lambda w: (w.reshape(-1)[:8].clone(), torch.arange(4, dtype=torch.uint8),
+                      torch.arange(w.shape[0] + 1, dtype=torch.int32), w.shape[0], w.shape[1])
+    compressed = llm.compress_state_dict(sd, compress=fake)
+    path = llm.save_compressed_state_dict(compressed, str(tmp_path / "model_compressed"))
+    back = llm.load_compressed_state_dict(path)
+    assert list(back.keys()) == list(compressed.keys())
+    for key, value in compressed.items():
+        if torch.is_tensor(value):
+            assert back[key].dtype == value.dtype and torch.equal(back[key], value), key
+        else:
+            assert type(back[key]) is int and back[key] == value, key
+    assert back["model.layers.0.self_attn.q_proj.c_3"] == 3 and back["model.layers.0.self_attn.q_proj.c_4"] == 4
+    # the file is what a plain weights-only torch.load gives, as the upstream runner does
+    plain = torch.load(path, weights_only=True)
+    assert isinstance(plain, OrderedDict) and plain["model.layers.0.self_attn.q_proj.c_4"] == 4
+
+
+@pytest.mark.gpu
+def test_saved_compressed_model_reloads_and_reproduces_the_logits(tmp_path):
+    torch.set_grad_enabled(False)
+    cfg = dict(n_layers=2, dim=256, hidden=688, n_heads=4, vocab=1000, max_len=64)
+    source, _ = llm.build_model(0.3, sparse=False, **cfg)
+    compressed_sd = llm.compress_state_dict(source.state_dict())
+    in_memory, _ = llm.build_model(0.3, sparse=False, **cfg)
+    llm.load_compressed_linears(in_memory, compressed_sd)
+    path = llm.save_compressed_state_dict(compressed_sd, str(tmp_path / "tiny_compressed"))
+    from_file, _ = llm.build_model(0.3, sparse=False, **cfg)
+    reloaded = llm.load_compressed_state_dict(path, device="cuda")
+    assert type(reloaded["model.layers.1.mlp.up_proj.c_3"]) is int
+    llm.load_compressed_linears(from_file, reloaded)
+    prompt = torch.randint(0, 1000, (1, 9), device="cuda")
+    pos = torch.arange(9, device="cuda")
+    a = in_memory(prompt, pos)
+    b = from_file(prompt, pos)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))  # bit for bit
+    want = source(prompt, pos).float()
+    assert torch.allclose(b.float(), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.gpu
+def test_engine_at_llama_7b_width_matches_the_module_path():
+    # the geometry of the end-to-end configuration (dim 4096, FFN 11008, 32 heads, vocab 32000) with
+    # three layers instead of 32: the fused engine on MACKO projections against the plain module
+    # forward on the same (pruned) dense weights
+    torch.set_grad_enabled(False)
+    cfg = dict(n_layers=3, dim=4096, hidden=11008, n_heads=32, vocab=32000, max_len=48)
+    for density in (0.5, 0.1):
+        reference, _ = llm.build_model(density, sparse=False, **cfg)
+        consumed, _ = llm.build_model(density, sparse=True, **cfg)
+        engine = llm.DecodeEngine(consumed, fuse=True)
+        prompt = torch.randint(0, 32000, (1, 6), device="cuda")
+        want = reference(prompt, torch.arange(6, device="cuda"))[0].float()
+        position = torch.zeros(1, dtype=torch.long, device="cuda")
+        spread = float(want.max() - want.min())
+        for i in range(6):
+            logits = engine.step(prompt[0, i:i + 1].clone(), position).float()
+            err = float((logits - want[i]).abs().max())
+            assert err <= 0.03 * max(spread, 1.0), (density, i, err, spread)
+            position.add_(1)
+        ids_graph, _ = llm.engine_decode(engine, prompt, 8, use_graph=True)
+        ids_eager, _ = llm.engine_decode(engine, prompt, 8, use_graph=False)
+        assert torch.equal(ids_graph, ids_eager)
+        del reference, consumed, engine
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.gpu
 def test_macko_linear_matches_dense_projection():
     torch.manual_seed(0)
