@@ -563,7 +563,7 @@ spmv_stream_kernel(const SpmvArgs a)
     // Entries [pos, seg_end) of the tile starting at entry `tb`, all in the current row: lanes
     // outside the segment are switched off, the first and last lane of the segment are masked.
     // A row that starts `q0` entries into its first lane shifts every address by -2*q0.
-    auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end) {
+    auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end, auto checked) {
         const int rel0 = pos - tb;
         const int rel1 = seg_end - tb;
         const int l0 = rel0 >> 3, q0 = rel0 & 7;
@@ -581,16 +581,12 @@ spmv_stream_kernel(const SpmvArgs a)
         row_addr = origin + (u32)__builtin_amdgcn_readlane((int)incl, kWave - 1);
         const int kmin = lane == l0 ? q0 : 0;
         const int kmax = (lane == l1 && q1 != 0) ? q1 : 8;
-#ifdef MACKO_NO_CHECK
-        if (active) lane_fma(vv, dd, base, index_constant<0>{}, kmin, kmax);
-#else
-        if (active) lane_fma(vv, dd, base, index_constant<1>{}, kmin, kmax);
-#endif
+        if (active) lane_fma(vv, dd, base, checked, kmin, kmax);
     };
 
-    auto finish_row = [&]() {
+    auto finish_row = [&](float total) {  // total: the row's sum where there is one vector
         if (NB == 1) {
-            store_row(r, wave_sum(acc0 + acc1));
+            store_row(r, total);
             acc0 = acc1 = 0.f;
         } else {
 #pragma unroll
@@ -626,16 +622,39 @@ spmv_stream_kernel(const SpmvArgs a)
             const int tile_end = tb + kTile;
             if (e0 <= tb && e1 >= tile_end) {  // the common case for rows longer than a tile
                 full_tile_pass(vj, dj);
-                if (e1 == tile_end) finish_row();
+                if (e1 == tile_end) finish_row(NB == 1 ? wave_sum(acc0 + acc1) : 0.f);
             } else {
                 const int lim = tile_end < s_end ? tile_end : s_end;
                 int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
                 while (pos < lim) {
                     const int seg_end = e1 < lim ? e1 : lim;
-                    segment_pass(vj, dj, tb, pos, seg_end);
                     const bool row_done = seg_end == e1;
+                    if constexpr (X_LDS && NB == 1) {
+                        // Entries behind a row's end are masked where they are read (CHECKED), which
+                        // costs a compare and a select per entry.  They can only matter if what they
+                        // read is Inf or NaN, and then the row's sum is not finite: so run unmasked,
+                        // and repeat the row's last piece masked in that rare case.  (A masked
+                        // entry that reads a finite number adds +-0 to a sum that started at +0.)
+                        const float keep0 = acc0, keep1 = acc1;
+                        const u32 keep_addr = row_addr;
+                        segment_pass(vj, dj, tb, pos, seg_end, index_constant<0>{});
+                        if (row_done) {
+                            float total = wave_sum(acc0 + acc1);
+                            const u32 bits = __builtin_bit_cast(u32, total);
+                            if (__builtin_expect((bits & 0x7f800000u) == 0x7f800000u, 0) && ((seg_end - tb) & 7) != 0) {
+                                acc0 = keep0;
+                                acc1 = keep1;
+                                row_addr = keep_addr;
+                                segment_pass(vj, dj, tb, pos, seg_end, index_constant<1>{});
+                                total = wave_sum(acc0 + acc1);
+                            }
+                            finish_row(total);
+                        }
+                    } else {
+                        segment_pass(vj, dj, tb, pos, seg_end, index_constant<1>{});
+                        if (row_done) finish_row(NB == 1 ? wave_sum(acc0 + acc1) : 0.f);
+                    }
                     pos = seg_end;
-                    if (row_done) finish_row();
                 }
             }
         });
