@@ -78,6 +78,17 @@ MACKO_API int macko_compress_f16_count(const void *dense, int32_t rows, int32_t 
                              int32_t *row_ptr, void *stream);
 
 /*
+ * Step 1 with the total handed over: as macko_compress_f16_count, and when row_ptr is complete
+ * the kernel also stores n = row_ptr[rows] to *total (a release store of system scope).  `total`
+ * is any int32 the GPU can write; given page-locked host memory that the caller has set to -1, a
+ * host thread can watch that word change instead of copying n back and synchronizing the stream,
+ * which takes several microseconds less.  total == NULL behaves as macko_compress_f16_count.
+ * No upstream counterpart (upstream's compressor runs on the host).
+ */
+MACKO_API int macko_compress_f16_count_total(const void *dense, int32_t rows, int32_t cols,
+                                             int32_t *row_ptr, int32_t *total, void *stream);
+
+/*
  * Compressor, step 2 of 2.  Fills values [P] (16-byte aligned) and deltas [P/2] (4-byte
  * aligned) from `dense` and the row_ptr produced by step 1; both arrays are fully written,
  * tail zero-filled, whatever they held before.  P must be ceil(row_ptr[rows]/8)*8.
@@ -129,6 +140,9 @@ MACKO_API int macko_spmv_f16_silu_mul_axpby(const void *values, const void *delt
  */
 MACKO_API int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols,
                             int32_t *row_ptr, void *stream);
+/* int8 twin of macko_compress_f16_count_total. */
+MACKO_API int macko_compress_i8_count_total(const void *dense, int32_t rows, int32_t cols,
+                                            int32_t *row_ptr, int32_t *total, void *stream);
 MACKO_API int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols,
                            const int32_t *row_ptr, void *values, void *deltas,
                            int64_t padded_entries, void *stream);

@@ -25,6 +25,7 @@ namespace {
 constexpr int kRowsPerBlock = 4;              // waves per workgroup, one row each
 constexpr int kBlock = kRowsPerBlock * kWave;
 constexpr int kNoColumn = (int)0x80000000;
+constexpr int kAhead = 4;                     // tiles of its row a wave keeps in flight
 
 // The two element formats.  A chunk is the 8 consecutive elements a lane handles per tile.
 struct Fp16Format {
@@ -37,6 +38,22 @@ struct Fp16Format {
     static __device__ __forceinline__ bool nonzero(u32 bits) { return (bits & 0x7fffu) != 0; }
     // what is stored: the element itself, a NaN as 0x7fff
     static __device__ __forceinline__ u32 stored(u32 bits) { return (bits & 0x7fffu) > 0x7c00u ? 0x7fffu : bits; }
+    // the 8 values of a full group from their stage words (value in the low half of each)
+    static __device__ __forceinline__ Chunk pack(const u32 (&e)[8])
+    {
+        Chunk v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = __builtin_amdgcn_perm(e[2 * k + 1], e[2 * k], 0x05040100u);
+        return v;
+    }
+    // a half is a NaN when its low 15 bits exceed 0x7c00: adding 0x03ff then carries into bit 15
+    static __device__ __forceinline__ bool any_nan(const Chunk &v)
+    {
+        u32 hit = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) hit |= ((v[w] & 0x7fff7fffu) + 0x03ff03ffu) & 0x80008000u;
+        return hit != 0;
+    }
 };
 struct Int8Format {
     typedef unsigned char Elem;
@@ -46,6 +63,18 @@ struct Int8Format {
     static __device__ __forceinline__ void put(Chunk &v, int i, u32 bits) { v[i >> 2] |= bits << (8 * (i & 3)); }
     static __device__ __forceinline__ bool nonzero(u32 bits) { return bits != 0; }
     static __device__ __forceinline__ u32 stored(u32 bits) { return bits; }
+    static __device__ __forceinline__ bool any_nan(const Chunk &) { return false; }
+    static __device__ __forceinline__ Chunk pack(const u32 (&e)[8])
+    {
+        Chunk v;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const u32 lo = __builtin_amdgcn_perm(e[4 * k + 1], e[4 * k], 0x0c0c0400u);
+            const u32 hi = __builtin_amdgcn_perm(e[4 * k + 3], e[4 * k + 2], 0x0c0c0400u);
+            v[k] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        return v;
+    }
 };
 
 // 8 consecutive elements of a row, zero beyond `cols`.  STREAM: the dense matrix will not be read
@@ -108,21 +137,31 @@ __global__ void __launch_bounds__(kBlock) count_rows_kernel(const typename F::El
     const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & (sizeof(Chunk) - 1)) == 0;
     int carry = -1;  // column of the last non-zero seen in earlier passes
     int mine = 0;
-    for (int c0 = 0; c0 < cols; c0 += kTile) {
-        const int col = c0 + lane * kChunk;
-        const Chunk v = load8<F, STREAM>(src, col, cols, vector_ok && col < cols);
-        const u32 nz = nonzero_bits<F>(v);
-        const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
-        int pass_last;
-        int p = previous_nonzero(own_last, carry, lane, pass_last);
+    // kAhead tiles of the row are in flight at any time: a wave walks its row alone, so what hides
+    // the memory latency is the depth of its own queue
+    Chunk ahead[kAhead];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (nz & (1u << i)) {
-                mine += 1 + ((col + i - p - 1) >> 4);
-                p = col + i;
-            }
+    for (int k = 0; k < kAhead; ++k) {
+        const int col = k * kTile + lane * kChunk;
+        ahead[k] = load8<F, STREAM>(src, col, cols, vector_ok && col < cols);
+    }
+    for (int c0 = 0; c0 < cols; c0 += kAhead * kTile) {
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            const int col = c0 + k * kTile + lane * kChunk;
+            if (c0 + k * kTile >= cols) break;  // wave-uniform
+            const Chunk v = ahead[k];
+            const int ncol = col + kAhead * kTile;
+            if (c0 + (k + kAhead) * kTile < cols) ahead[k] = load8<F, STREAM>(src, ncol, cols, vector_ok && ncol < cols);
+            const u32 nz = nonzero_bits<F>(v);
+            const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
+            int pass_last;
+            const int p = previous_nonzero(own_last, carry, lane, pass_last);
+            // every non-zero is an entry; padding entries can only stand in front of the first
+            // non-zero of my 8 columns (the others follow their predecessor within 8 columns)
+            if (nz) mine += __builtin_popcount(nz) + ((col + __builtin_ctz(nz) - p - 1) >> 4);
+            carry = pass_last > carry ? pass_last : carry;
         }
-        carry = pass_last > carry ? pass_last : carry;
     }
     int total = wave_sum_int(mine);
     if (F::kKeepTrailing) total += (cols - 1 - carry) >> 4;  // padding entries at carry+16, carry+32, ... < cols
@@ -130,54 +169,102 @@ __global__ void __launch_bounds__(kBlock) count_rows_kernel(const typename F::El
 }
 
 // row_ptr[0] = 0, row_ptr[r+1] = counts[0] + ... + counts[r].  `counts` aliases row_ptr + 1.
-// One workgroup; each thread owns a contiguous slice.
-__global__ void __launch_bounds__(1024) scan_rows_kernel(int *__restrict__ row_ptr, int rows)
+// One workgroup walks the rows in slices of kScanSlice: the slice comes into LDS through
+// coalesced loads that are all in flight together, each thread sums and scans the kScanPer
+// consecutive rows it owns there, and the slice goes back out coalesced.
+constexpr int kScanPer = 8;
+constexpr int kScanSlice = 1024 * kScanPer;
+__global__ void __launch_bounds__(1024) scan_rows_kernel(int *__restrict__ row_ptr, int rows, int *total_out)
 {
+    __shared__ int slice[kScanSlice + kScanSlice / 32];  // one word of padding per 32: consecutive owners, different banks
     __shared__ int wave_totals[16];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
-    const int per = (rows + 1023) / 1024;
-    const int begin = tid * per < rows ? tid * per : rows;
-    const int end = begin + per < rows ? begin + per : rows;
     int *counts = row_ptr + 1;
-    int sum = 0;
-    for (int i = begin; i < end; ++i) sum += counts[i];
-    const int incl = wave_scan_inclusive(sum);
-    if (lane == kWave - 1) wave_totals[wave] = incl;
-    __syncthreads();
-    int base = incl - sum;
-    for (int w = 0; w < wave; ++w) base += wave_totals[w];
-    for (int i = begin; i < end; ++i) {
-        base += counts[i];
-        counts[i] = base;
+    int running = 0;  // sum of all earlier slices
+    auto at = [](int i) { return i + (i >> 5); };
+    for (int s0 = 0; s0 < rows; s0 += kScanSlice) {
+        int v[kScanPer];
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) {
+            const int i = s0 + j * 1024 + tid;
+            v[j] = i < rows ? counts[i] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) slice[at(j * 1024 + tid)] = v[j];
+        __syncthreads();
+        int sum = 0;
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) {
+            sum += slice[at(tid * kScanPer + j)];
+            v[j] = sum;
+        }
+        const int incl = wave_scan_inclusive(sum);
+        if (lane == kWave - 1) wave_totals[wave] = incl;
+        __syncthreads();
+        int base = running + incl - sum;
+        int slice_total = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            const int t = wave_totals[w];
+            base += w < wave ? t : 0;
+            slice_total += t;
+        }
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) slice[at(tid * kScanPer + j)] = base + v[j];
+        running += slice_total;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) {
+            const int i = s0 + j * 1024 + tid;
+            if (i < rows) counts[i] = slice[at(j * 1024 + tid)];
+        }
+        __syncthreads();  // the slice and the wave totals are reused
     }
-    if (tid == 0) row_ptr[0] = 0;
+    if (tid == 0) {
+        row_ptr[0] = 0;
+        // for a host thread that waits for this word to change rather than for the stream
+        if (total_out != nullptr) __hip_atomic_store(total_out, running, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
-// Packs the low nibbles of 8 staged entries (bits 16..19 of each word) into one delta word.
+// Packs the nibbles of 8 staged entries (bits 16..19 of each word, bits 20..23 zero) into one delta
+// word: byte 2 of four words at a time into one register, neighbouring bytes folded into one byte.
 __device__ __forceinline__ u32 pack_nibbles(const u32 (&e)[8])
 {
-    u32 w = 0;
+    u32 folded[2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) w |= ((e[i] >> 16) & 15u) << (4 * i);
-    return w;
+    for (int h = 0; h < 2; ++h) {
+        const u32 a = __builtin_amdgcn_perm(e[4 * h + 1], e[4 * h], 0x0c0c0602u);      // n0 | n1 << 8
+        const u32 b = __builtin_amdgcn_perm(e[4 * h + 3], e[4 * h + 2], 0x0c0c0602u);  // n2 | n3 << 8
+        const u32 four = __builtin_amdgcn_perm(b, a, 0x05040100u);                     // n0, n1, n2, n3 in bytes
+        folded[h] = four | (four >> 4);  // byte 0 = n0 | n1 << 4, byte 2 = n2 | n3 << 4
+    }
+    return __builtin_amdgcn_perm(folded[1], folded[0], 0x06040200u);
 }
 
-// Orders this wave's LDS writes before its later LDS reads (the staging area is private to
-// the wave, so no workgroup barrier is involved).
+// Orders this wave's LDS writes before its later LDS reads by other lanes.  The staging area is
+// private to the wave and a wave's LDS operations are carried out in the order issued, so this is
+// a matter of instruction order only: fences of wavefront scope, which wait for nothing (a wider
+// scope would also wait for the row's loads in flight and the stores on their way out).
 __device__ __forceinline__ void wave_lds_fence()
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Pass 2.  The wave stages the entries of its row in LDS at the offset they have inside their
 // 8-entry group of the output, so that every complete group leaves as one 16-byte store of
 // values and one 4-byte store of nibbles.  Groups cut by a row boundary are shared with the
-// neighbouring row's wave: their values go out as 2-byte stores and their nibbles are OR-ed
-// into the (zeroed) delta word.  `deltas` must be zero on entry; `values` need not be.
+// neighbouring row's wave: their values go out as 2-byte stores and their nibbles as bytes.  A
+// byte holds two nibbles; where a row ends on an odd entry its last nibble shares a byte with the
+// first nibble of the next non-empty row.  That byte is written by the earlier row's wave, which
+// works the later row's first nibble out for itself from that row's first 16 columns (the column
+// of its first non-zero, or 15 for a padding entry); the later row's wave leaves the byte alone.
+// So every byte of `deltas` and every element of `values` has exactly one writer, and neither
+// array needs to be cleared beforehand.
 template <typename F, bool STREAM>
 __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Elem *__restrict__ dense, int rows,
                                                            int cols, const int *__restrict__ row_ptr,
@@ -187,7 +274,28 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Ele
     typedef typename F::Elem Elem;
     typedef typename F::Chunk Chunk;
     constexpr int kStage = kTile + 8;  // a tile's entries plus the carried part of a group
-    __shared__ u32 stage_all[kRowsPerBlock][kStage];
+    __shared__ __attribute__((aligned(16))) u32 stage_all[kRowsPerBlock][kStage + kWave];  // + a spare word per lane
+    // gap_table[m]: the 8 nibbles of a lane whose non-zero columns are the set bits of m, as far as
+    // they can be told from m alone: 15 where there is no non-zero, the distance to the previous
+    // set bit less one for a non-zero, and 0 for the first non-zero, whose distance reaches back
+    // into earlier lanes and is put in by the lane itself
+    __shared__ u32 gap_table[256];
+    static_assert(kBlock == 256, "one table entry per thread");
+    {
+        const u32 m = threadIdx.x;
+        u32 word = 0;
+        int previous = -1;
+        for (int i = 0; i < 8; ++i) {
+            u32 nib = 15u;
+            if ((m >> i) & 1u) {
+                nib = previous < 0 ? 0u : (u32)(i - previous - 1);
+                previous = i;
+            }
+            word |= nib << (4 * i);
+        }
+        gap_table[m] = word;
+    }
+    __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = uniform(threadIdx.x >> 6);
     const int row = blockIdx.x * kRowsPerBlock + wave;
@@ -196,11 +304,38 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Ele
     const int e1 = row_ptr[row + 1];
     u32 *stage = stage_all[wave];
     Chunk *value_groups = reinterpret_cast<Chunk *>(values);
+    unsigned char *delta_bytes = reinterpret_cast<unsigned char *>(delta_words);
 
-    if (row == rows - 1) {  // the unused tail of the last 8-entry group
+    if (row == rows - 1) {  // the unused tail of the last 8-entry group (an odd e1's byte has its owner)
         for (int i = e1 + lane; i < padded; i += kWave) values[i] = 0;
+        for (int i = ((e1 + 1) >> 1) + lane; i < (padded >> 1); i += kWave) delta_bytes[i] = 0;
     }
     if (e0 == e1) return;
+
+    // The first nibble behind my row, wanted if my last entry is the low half of a byte: asked for
+    // now, on the guess that the next row is not empty, and looked at when my row is done.
+    const bool shares_last_byte = (e1 & 1) != 0;
+    const bool probe_lane = lane < 16 && lane < cols;
+    int next_end = e1;
+    u32 next_probe = 0;
+    if (shares_last_byte && row + 1 < rows) {
+        next_end = row_ptr[row + 2];
+        if (probe_lane) next_probe = dense[(size_t)(row + 1) * (size_t)cols + lane];
+    }
+    auto first_nibble_behind = [&]() -> u32 {
+        int r2 = row + 1;
+        if (r2 >= rows) return 0u;  // my row holds the last entry: the rest of the byte is padding
+        if (next_end == e1) {       // empty rows behind mine: walk on to the next one that is not
+            do {
+                ++r2;
+            } while (r2 < rows && row_ptr[r2 + 1] == e1);
+            if (r2 >= rows) return 0u;
+            next_probe = probe_lane ? (u32)dense[(size_t)r2 * (size_t)cols + lane] : 0u;
+        }
+        // a row with entries whose first 16 columns are zero starts with the padding entry of column 15
+        const unsigned long long m = __ballot(probe_lane && F::nonzero(next_probe));
+        return m ? (u32)__builtin_ctzll(m) : 15u;
+    };
 
     const Elem *src = dense + (size_t)row * (size_t)cols;
     const bool vector_ok = (reinterpret_cast<uintptr_t>(src) & (sizeof(Chunk) - 1)) == 0;
@@ -212,8 +347,8 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Ele
     int carry = -1;
 
     // writes out groups [0, n_groups) of the stage; group g holds entries [a, b) with
-    // a = lo for group 0 and b = hi - 8g for a last, incomplete group
-    auto flush = [&](int n_groups) {
+    // a = lo for group 0 and b = hi - 8g for a last, incomplete group (which ends the row)
+    auto flush = [&](int n_groups, u32 nibble_behind) {
         for (int g = lane; g < n_groups; g += kWave) {
             u32 e[8];
 #pragma unroll
@@ -222,80 +357,99 @@ __global__ void __launch_bounds__(kBlock) fill_rows_kernel(const typename F::Ele
             const int b = hi - 8 * g < 8 ? hi - 8 * g : 8;
             const int out = (base >> 3) + g;
             if (a == 0 && b == 8) {
-                Chunk v = {};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) F::put(v, i, e[i] & 0xffffu);
-                value_groups[out] = v;
+                value_groups[out] = F::pack(e);
                 delta_words[out] = pack_nibbles(e);
             } else {
-                u32 keep = 0;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (i >= a && i < b) {
-                        values[8 * (size_t)out + i] = (Elem)e[i];
-                        keep |= 15u << (4 * i);
+                for (int i = 0; i < 8; ++i)
+                    if (i >= a && i < b) values[8 * (size_t)out + i] = (Elem)e[i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool low_mine = 2 * j >= a && 2 * j < b;
+                    const bool high_mine = 2 * j + 1 >= a && 2 * j + 1 < b;
+                    // low nibble mine: my byte, whoever the high nibble belongs to
+                    if (low_mine) {
+                        const u32 low = (e[2 * j] >> 16) & 15u;
+                        const u32 high = high_mine ? (e[2 * j + 1] >> 16) & 15u : nibble_behind;
+                        delta_bytes[4 * (size_t)out + j] = (unsigned char)(low | (high << 4));
                     }
                 }
-                atomicOr(&delta_words[out], pack_nibbles(e) & keep);
             }
         }
     };
 
-    Chunk next = load8<F, STREAM>(src, lane * kChunk, cols, vector_ok && lane * kChunk < cols);
-    for (int c0 = 0; c0 < cols; c0 += kTile) {
-        const int col = c0 + lane * kChunk;
-        const Chunk v = next;
-        if (c0 + kTile < cols) {
-            const int ncol = col + kTile;
-            next = load8<F, STREAM>(src, ncol, cols, vector_ok && ncol < cols);
-        }
-        const u32 nz = nonzero_bits<F>(v);
-        const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
-        int pass_last;
-        int p = previous_nonzero(own_last, carry, lane, pass_last);
-        carry = pass_last > carry ? pass_last : carry;
-        // which of my 8 columns store an entry, and with which nibble
-        u32 entry_bits = 0;
-        u32 nibbles = 0;
+    // kAhead tiles of the row in flight, as in pass 1
+    Chunk ahead[kAhead];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int x = col + i;
-            const int dist = x - p;
-            const bool is_nz = (nz >> i) & 1u;
-            const bool is_entry = x < cols && (is_nz || (dist & 15) == 0);
-            const u32 nib = is_nz ? (u32)(dist - 1) & 15u : 15u;
-            entry_bits |= (is_entry ? 1u : 0u) << i;
-            nibbles |= nib << (4 * i);
-            p = is_nz ? x : p;
-        }
-        const int mine = __builtin_popcount(entry_bits);
-        const int incl = wave_scan_inclusive(mine);
-        const int produced = __builtin_amdgcn_readlane(incl, kWave - 1);
-        // entries past e1 are padding entries behind the row's last non-zero: not stored
-        const int room = e1 - (base + hi);
-        const int n_new = produced < room ? produced : room;
-        int slot = incl - mine;
+    for (int k = 0; k < kAhead; ++k) {
+        const int col = k * kTile + lane * kChunk;
+        ahead[k] = load8<F, STREAM>(src, col, cols, vector_ok && col < cols);
+    }
+    bool row_done = false;
+    for (int c0 = 0; c0 < cols && !row_done; c0 += kAhead * kTile) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if ((entry_bits & (1u << i)) && slot < n_new) {
-                stage[hi + slot] = F::stored(F::at(v, i)) | (((nibbles >> (4 * i)) & 15u) << 16);
-                ++slot;
+        for (int k = 0; k < kAhead; ++k) {
+            if (row_done || c0 + k * kTile >= cols) break;  // wave-uniform
+            const int col = c0 + k * kTile + lane * kChunk;
+            const Chunk v = ahead[k];
+            const int ncol = col + kAhead * kTile;
+            if (c0 + (k + kAhead) * kTile < cols) ahead[k] = load8<F, STREAM>(src, ncol, cols, vector_ok && ncol < cols);
+            const u32 nz = nonzero_bits<F>(v);
+            const int own_last = nz ? col + 31 - __builtin_clz(nz) : kNoColumn;
+            int pass_last;
+            int p = previous_nonzero(own_last, carry, lane, pass_last);
+            carry = pass_last > carry ? pass_last : carry;
+            // Non-zeros are entries.  A padding entry stands at p + 16, p + 32, ...: among my 8
+            // columns at most one, and only in front of my first non-zero (behind it the previous
+            // non-zero is less than 8 columns away).
+            const int pad_at = p + (((col - p + 15) >> 4) << 4) - col;  // >= 0, my column index of it
+            const int first_nz = nz ? __builtin_ctz(nz) : 8;
+            const bool has_pad = pad_at < first_nz && col + pad_at < cols;
+            const u32 entry_bits = nz | (has_pad ? 1u << pad_at : 0u);
+            u32 nibbles = gap_table[nz];
+            if (nz) nibbles |= ((u32)(col + first_nz - p - 1) & 15u) << (4 * first_nz);
+            const int mine = __builtin_popcount(entry_bits);
+            const int incl = wave_scan_inclusive(mine);
+            const int produced = __builtin_amdgcn_readlane(incl, kWave - 1);
+            // entries past e1 are padding entries behind the row's last non-zero: not stored
+            const int room = e1 - (base + hi);
+            const int n_new = produced < room ? produced : room;
+            // Those dropped entries are whole lanes: behind the row's last non-zero a lane holds at
+            // most its one padding entry, and the lane of the last non-zero has its padding entry
+            // in front of it.  So a lane keeps all of its entries or none.
+            const int slot = incl - mine;
+            const u32 kept = slot < n_new ? entry_bits : 0u;
+            Chunk vs = v;
+            if (__builtin_expect(__ballot(F::any_nan(v)) != 0ull, 0)) {  // NaNs are stored in one form
+                vs = Chunk{};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) F::put(vs, i, F::stored(F::at(v, i)));
             }
-        }
-        hi += n_new;
-        wave_lds_fence();
-        const bool row_done = base + hi == e1;
-        const int n_groups = row_done ? (hi + 7) >> 3 : hi >> 3;
-        flush(n_groups);
-        if (row_done) break;
-        if (n_groups > 0) {  // carry the incomplete group to the front of the stage
-            const int rest = hi & 7;
-            const u32 moved = lane < rest ? stage[8 * n_groups + lane] : 0u;
+            // every lane writes all 8 of its columns, no branches: what is not kept goes to a word
+            // of the lane's own behind the stage
+            const int first_index = hi + slot;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool take = ((kept >> i) & 1u) != 0;
+                const int rank = __builtin_popcount(kept & ((1u << i) - 1u));
+                const u32 word = F::at(vs, i) | (((nibbles >> (4 * i)) & 15u) << 16);
+                stage[take ? first_index + rank : kStage + lane] = word;
+            }
+            hi += n_new;
             wave_lds_fence();
-            if (lane < rest) stage[lane] = moved;
-            base += 8 * n_groups;
-            lo = 0;
-            hi = rest;
+            row_done = base + hi == e1;
+            const int n_groups = row_done ? (hi + 7) >> 3 : hi >> 3;
+            flush(n_groups, row_done && shares_last_byte ? first_nibble_behind() : 0u);
+            if (row_done) break;
+            if (n_groups > 0) {  // carry the incomplete group to the front of the stage
+                const int rest = hi & 7;
+                const u32 moved = lane < rest ? stage[8 * n_groups + lane] : 0u;
+                wave_lds_fence();
+                if (lane < rest) stage[lane] = moved;
+                base += 8 * n_groups;
+                lo = 0;
+                hi = rest;
+            }
         }
     }
 }
@@ -358,7 +512,7 @@ bool streams_past_cache(int32_t rows, int32_t cols)
 }
 
 template <typename F>
-int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr, void *stream)
+int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr, int32_t *total, void *stream)
 {
     typedef typename F::Elem Elem;
     if (rows < 0 || cols < 0 || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
@@ -379,7 +533,8 @@ int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_p
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, s, row_ptr, rows);
+    if (reinterpret_cast<uintptr_t>(total) & 3) return MACKO_E_INVALID_ARGUMENT;
+    hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, s, row_ptr, rows, total);
     return (int)hipGetLastError();
 }
 
@@ -399,10 +554,7 @@ int compress_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *
         (reinterpret_cast<uintptr_t>(deltas) & 3))
         return MACKO_E_INVALID_ARGUMENT;
     hipStream_t s = as_stream(stream);
-    // row-boundary nibbles are OR-ed in, so the nibble array starts from zero
-    hipError_t e = hipMemsetAsync(deltas, 0, (size_t)padded_entries / 2, s);
-    if (e != hipSuccess) return (int)e;
-    if (rows == 0) return (int)hipMemsetAsync(values, 0, (size_t)padded_entries * sizeof(Elem), s);
+    if (rows == 0) return MACKO_E_INVALID_ARGUMENT;  // entries without rows
     const dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock);
     if (streams_past_cache<Elem>(rows, cols))
         hipLaunchKernelGGL((fill_rows_kernel<F, true>), grid, dim3(kBlock), 0, s, (const Elem *)dense, rows, cols,
@@ -419,7 +571,7 @@ int compress_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *
 extern "C" int macko_compress_f16_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
                                         void *stream)
 {
-    return macko::compress_count<macko::Fp16Format>(dense, rows, cols, row_ptr, stream);
+    return macko::compress_count<macko::Fp16Format>(dense, rows, cols, row_ptr, nullptr, stream);
 }
 
 extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,
@@ -429,10 +581,22 @@ extern "C" int macko_compress_f16_fill(const void *dense, int32_t rows, int32_t 
                                                    stream);
 }
 
+extern "C" int macko_compress_f16_count_total(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                              int32_t *total, void *stream)
+{
+    return macko::compress_count<macko::Fp16Format>(dense, rows, cols, row_ptr, total, stream);
+}
+
+extern "C" int macko_compress_i8_count_total(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
+                                             int32_t *total, void *stream)
+{
+    return macko::compress_count<macko::Int8Format>(dense, rows, cols, row_ptr, total, stream);
+}
+
 extern "C" int macko_compress_i8_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_ptr,
                                        void *stream)
 {
-    return macko::compress_count<macko::Int8Format>(dense, rows, cols, row_ptr, stream);
+    return macko::compress_count<macko::Int8Format>(dense, rows, cols, row_ptr, nullptr, stream);
 }
 
 extern "C" int macko_compress_i8_fill(const void *dense, int32_t rows, int32_t cols, const int32_t *row_ptr,

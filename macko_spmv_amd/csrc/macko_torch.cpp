@@ -14,6 +14,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include <chrono>
 #include <tuple>
 
 #include "macko_decode.h"
@@ -109,10 +110,29 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_on_dev
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     const bool int8 = M.dtype() == at::kChar;
     at::Tensor row_ptr = at::empty({rows + 1}, M.options().dtype(at::kInt));
-    check_rc((int8 ? macko_compress_i8_count : macko_compress_f16_count)(
-                 M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(), (void *)stream),
+    // The entry count sizes the outputs, so the host has to wait for it.  The count pass stores it
+    // into a page-locked word of this thread's, which the thread watches for a short while (a
+    // matrix of a few thousand rows and columns is through in about ten microseconds, and the
+    // store is seen much sooner than a stream synchronization returns); for anything longer it
+    // falls back to waiting for the stream.
+    // (never released: at thread or process exit the runtime it would go back to may be gone already)
+    thread_local at::Tensor *total_word =
+        new at::Tensor(at::empty({1}, at::TensorOptions().dtype(at::kInt).pinned_memory(true)));
+    volatile int *total = total_word->data_ptr<int>();
+    *total = -1;
+    check_rc((int8 ? macko_compress_i8_count_total : macko_compress_f16_count_total)(
+                 M.data_ptr(), (int32_t)rows, (int32_t)cols, row_ptr.data_ptr<int>(), total_word->data_ptr<int>(),
+                 (void *)stream),
              "compress (count)");
-    const int64_t n = row_ptr[rows].item<int>();  // one 4-byte read-back; sizes the outputs
+    const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(200);
+    while (__atomic_load_n(total, __ATOMIC_ACQUIRE) < 0 && std::chrono::steady_clock::now() < give_up) {
+    }
+    if (__atomic_load_n(total, __ATOMIC_ACQUIRE) < 0) {
+        const hipError_t e = hipStreamSynchronize(stream);
+        TORCH_CHECK(e == hipSuccess, "macko_spmv: compress (waiting for the entry count): ", hipGetErrorString(e));
+    }
+    const int64_t n = __atomic_load_n(total, __ATOMIC_ACQUIRE);
+    TORCH_CHECK(n >= 0, "macko_spmv: compress: the count pass did not deliver the entry count");
     const int64_t padded = (n + 7) / 8 * 8;
     at::Tensor values = at::empty({padded}, M.options());
     at::Tensor deltas = at::empty({padded / 2}, M.options().dtype(at::kByte));
