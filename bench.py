@@ -551,27 +551,61 @@ def main():
             batched_cases.append(entry)
             log("batched:", entry)
 
-    # ---- the compressor: whole compress() call (count pass, read-back of the total, fill pass) -----
+    # ---- the compressor: the whole compress() call (count pass, wait for the total, allocation,
+    #      fill pass) and, beside it, the kernels alone (the C ABI's two steps launched back to
+    #      back on outputs that exist already) ----------------------------------------------------
     compress_cases = []
     if not args.no_compress:
+        hip = ctypes.CDLL(mk.HIP_LIBRARY_PATH)
+        vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+        hip.macko_compress_f16_count.argtypes = [vp, i32, i32, vp, vp]
+        hip.macko_compress_f16_fill.argtypes = [vp, i32, i32, vp, vp, vp, i64, vp]
         for c in cases:
             if c["density"] != 0.5:
                 continue
             W = c["W"]
+            R, C = c["rows"], c["cols"]
             for _ in range(2):
                 comp = mk.compress(W)
             torch.cuda.synchronize()
-            reps = 5
+            reps = 10
             t0 = time.perf_counter()
             for _ in range(reps):
                 comp = mk.compress(W)
             torch.cuda.synchronize()
             dt = (time.perf_counter() - t0) / reps
+            P = comp[0].numel()
+            stream = torch.cuda.current_stream().cuda_stream
+            row_ptr = torch.empty_like(comp[2])
+            values = torch.empty_like(comp[0])
+            deltas = torch.empty_like(comp[1])
+
+            def kernels():
+                rc = hip.macko_compress_f16_count(W.data_ptr(), R, C, row_ptr.data_ptr(), stream)
+                rc = rc or hip.macko_compress_f16_fill(W.data_ptr(), R, C, row_ptr.data_ptr(), values.data_ptr(),
+                                                       deltas.data_ptr(), P, stream)
+                if rc:
+                    raise RuntimeError(f"compress through the C ABI failed with code {rc}")
+
+            kernels()
+            torch.cuda.synchronize()
+            if not (torch.equal(values, comp[0]) and torch.equal(deltas, comp[1]) and torch.equal(row_ptr, comp[2])):
+                raise RuntimeError("compress through the C ABI differs from compress()")
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                kernels()
+            e1.record()
+            torch.cuda.synchronize()
+            dt_kernels = e0.elapsed_time(e1) * 1e-3 / reps
             # both passes read the dense matrix; the second writes values, nibbles; row_ptr is written twice
-            nbytes = 2 * dense_bytes(c["rows"], c["cols"]) + 2.5 * comp[0].numel() + 8 * (c["rows"] + 1)
-            entry = {"shape": f"{c['rows']}x{c['cols']}", "density": c["density"], "us": round(dt * 1e6, 1),
+            nbytes = 2 * dense_bytes(R, C) + 2.5 * P + 8 * (R + 1)
+            entry = {"shape": f"{R}x{C}", "density": c["density"], "us": round(dt * 1e6, 1),
                      "gbps": round(nbytes / dt / 1e9, 1),
-                     "pct_hbm_peak": round(100 * nbytes / dt / 1e9 / HBM_PEAK_GBPS, 1)}
+                     "pct_hbm_peak": round(100 * nbytes / dt / 1e9 / HBM_PEAK_GBPS, 1),
+                     "kernels_us": round(dt_kernels * 1e6, 1),
+                     "kernels_gbps": round(nbytes / dt_kernels / 1e9, 1),
+                     "kernels_pct_hbm_peak": round(100 * nbytes / dt_kernels / 1e9 / HBM_PEAK_GBPS, 1)}
             compress_cases.append(entry)
             log("compress:", entry)
 

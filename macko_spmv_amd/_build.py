@@ -227,6 +227,20 @@ def build_bench(verbose=False):
     return out
 
 
+def build_devtools(verbose=False):
+    """Development tools, not part of the product and never loaded by it: a tracing build of the
+    HIP library (phase stamps and launch-shape overrides, -DMACKO_DEV_HOOKS) and phase_trace,
+    the program that prints per-wave phase tables from it.  Both land in macko_spmv_amd/devtools/."""
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "devtools")
+    lib = os.path.join(here, "libmacko_hip_trace.so")
+    tool = os.path.join(here, "phase_trace")
+    _run([_hipcc(), *_DEVICE_FLAGS, "-DMACKO_DEV_HOOKS", "-fPIC", "-shared",
+          *[os.path.join(_CSRC, s) for s in HIP_SOURCES], "-o", lib], verbose)
+    _run([_hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", os.path.join(here, "phase_trace.hip"),
+          "-ldl", "-o", tool], verbose)
+    return lib, tool
+
+
 def build_all(verbose=False):
     if os.path.exists(stamp_path()):
         os.remove(stamp_path())
@@ -238,5 +252,6 @@ def build_all(verbose=False):
 
 
 if __name__ == "__main__":
-    for path in build_all(verbose="-q" not in sys.argv):
+    build = build_devtools if "--devtools" in sys.argv else build_all
+    for path in build(verbose="-q" not in sys.argv):
         print("built", path)
