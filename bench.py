@@ -232,39 +232,49 @@ def load_bench_library():
 
 
 def timed_steps(torch, mk, cases, steps, warmup):
-    """K steps replayed from graphs on a side stream; returns seconds for exactly `steps` steps."""
+    """K steps replayed from graphs on a side stream; returns seconds for exactly `steps` steps.
+
+    Steps alternate between two copies of every matrix.  A graph holds enough steps for about 48
+    launches (at least two steps), so that the time between two replays, which belongs to the
+    host, stays small beside the launches of one replay also where a step is only two launches."""
     def step(copy):
         for c in cases:
             mk.multiply(c["copies"][copy], c["x"])
 
-    def two_steps():
-        step(0)
-        step(1)
+    per_graph = max(2, -(-48 // len(cases)))
+    per_graph += per_graph % 2  # both copies equally often
+
+    def many_steps():
+        for j in range(per_graph):
+            step(j % 2)
 
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(stream):
-        two_steps()
+        step(0)
+        step(1)
         stream.synchronize()
-        g2 = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g2, stream=stream):
-            two_steps()
-        g1 = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g1, stream=stream):
-            step(0)
-        for _ in range(warmup // 2):
-            g2.replay()
-        if warmup % 2:
-            g1.replay()
+        g_many = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_many, stream=stream):
+            many_steps()
+        g1 = [torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()]
+        for copy in (0, 1):
+            with torch.cuda.graph(g1[copy], stream=stream):
+                step(copy)
+
+        def run(n):
+            for _ in range(n // per_graph):
+                g_many.replay()
+            for j in range(n % per_graph):
+                g1[j % 2].replay()
+
+        run(warmup)
         stream.synchronize()
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         start.record(stream)
-        for _ in range(steps // 2):
-            g2.replay()
-        if steps % 2:
-            g1.replay()
+        run(steps)
         end.record(stream)
         end.synchronize()
         torch.cuda.synchronize()
@@ -319,7 +329,7 @@ def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with
 
     # per-case timing, each over >= 1 GB of distinct copies
     per_case = []
-    for c in cases:
+    for c in cases if case_replays > 0 else []:
         n_sparse = max(2, min(256, int(1.0e9 // c["bytes"]) + 1))
         copies = c["copies"] + [clone_compressed(c["copies"][0]) for _ in range(n_sparse - 2)]
         t_sparse, _ = time_graph(torch, lambda: [mk.multiply(cc, c["x"]) for cc in copies], case_replays)
@@ -458,7 +468,9 @@ def main():
     ap.add_argument("--no-int8", action="store_true", help="skip the int8-values variant timing")
     ap.add_argument("--no-batched", action="store_true", help="skip the batched-product timing")
     ap.add_argument("--no-yardstick", action="store_true", help="skip the streaming-read yardstick")
-    ap.add_argument("--case-replays", type=int, default=20, help="graph replays per single-case timing")
+    ap.add_argument("--case-replays", type=int, default=20,
+                    help="graph replays per single-case timing (0: no per-case timings, so that a kernel trace of "
+                         "the run holds the timed steps' mix of launches and little else)")
     ap.add_argument("--suite", choices=sorted(WORKLOADS), default="llama",
                     help="the workload `value` is measured on (llama = the headline workload)")
     ap.add_argument("--also", default="large,skew,fewrows",
