@@ -222,6 +222,51 @@ class ReadYardstick:
         return t / copies
 
 
+def timed_steps_concurrent(torch, mk, cases, steps, warmup, n_streams):
+    """The same steps with their launches dealt round-robin to `n_streams` streams inside the
+    graphs: the multiplies of a step are independent, so one launch's last waves and the next
+    launch's prologue may overlap.  Returns seconds per step.  A figure reported beside the
+    headline, never as it: the headline times launches one after the other."""
+    per_graph = max(2, -(-48 // len(cases)))
+    per_graph += per_graph % 2
+    main = torch.cuda.Stream()
+    side = [torch.cuda.Stream() for _ in range(n_streams)]
+    main.wait_stream(torch.cuda.current_stream())
+
+    def many_steps():
+        for s in side:
+            s.wait_stream(main)
+        k = 0
+        for j in range(per_graph):
+            for c in cases:
+                with torch.cuda.stream(side[k % n_streams]):
+                    mk.multiply(c["copies"][j % 2], c["x"])
+                k += 1
+        for s in side:
+            main.wait_stream(s)
+
+    with torch.cuda.stream(main):
+        many_steps()
+        main.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=main):
+            many_steps()
+        replays = max(1, steps // per_graph)
+        for _ in range(max(1, warmup // per_graph)):
+            graph.replay()
+        main.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record(main)
+        for _ in range(replays):
+            graph.replay()
+        end.record(main)
+        end.synchronize()
+        torch.cuda.synchronize()
+    torch.cuda.current_stream().wait_stream(main)
+    return start.elapsed_time(end) * 1e-3 / (replays * per_graph)
+
+
 def load_bench_library():
     from macko_spmv_amd import _build
 
@@ -282,7 +327,8 @@ def timed_steps(torch, mk, cases, steps, warmup):
     return start.elapsed_time(end) * 1e-3
 
 
-def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with_dense=True, keep_dense=False):
+def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with_dense=True, keep_dense=False,
+                  concurrent_streams=0):
     """Builds a workload, checks what is about to be timed against the dense product, times `steps`
     steps of it and every case on its own.  Returns (summary dict, cases) -- `cases` keep their
     inputs only when keep_dense is set."""
@@ -326,6 +372,16 @@ def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with
     launch_us = elapsed_s * 1e6 / (steps * n_launch)
     log(f"[{suite}] timed region: {steps} steps, {elapsed_s * 1e3 / steps:.4f} ms/step, {gbps:.1f} GB/s effective, "
         f"{launch_us:.2f} us per launch on average")
+
+    concurrent = None
+    if concurrent_streams > 1:
+        step_s = timed_steps_concurrent(torch, mk, cases, steps, warmup, concurrent_streams)
+        concurrent = {"streams": concurrent_streams, "ms_per_step": round(step_s * 1e3, 5),
+                      "value": round(step_bytes / step_s / 1e9, 2), "unit": "GB/s",
+                      "frac_of_hbm_peak": round(step_bytes / step_s / 1e9 / HBM_PEAK_GBPS, 4),
+                      "what": "the same steps with their launches dealt to several streams inside the graphs, so "
+                              "that independent launches may overlap; beside the headline, not part of it"}
+        log(f"[{suite}] with {concurrent_streams} streams: {concurrent['ms_per_step']} ms/step, {concurrent['value']} GB/s")
 
     # per-case timing, each over >= 1 GB of distinct copies
     per_case = []
@@ -376,6 +432,7 @@ def measure_suite(torch, mk, suite, steps, warmup, yardstick, case_replays, with
         # against the faster of torch.matmul(W, x) and torch.matmul(x[None], W.T) per case
         "speedup_vs_best_dense_fp16": {"d0.5": mean_speedup(0.5, "speedup_vs_best_dense"),
                                        "d0.1": mean_speedup(0.1, "speedup_vs_best_dense")},
+        "launches_overlapped": concurrent,
         "cases": per_case,
     }
     if yardstick is not None and per_case:
@@ -477,6 +534,9 @@ def main():
                     help="comma-separated workloads measured in the same run and reported under `suites` "
                          "('' for none)")
     ap.add_argument("--also-steps", type=int, default=40, help="timed steps of each workload under `suites`")
+    ap.add_argument("--overlap-streams", type=int, default=4,
+                    help="also time the headline workload's steps with their launches dealt to this many streams "
+                         "(reported under `launches_overlapped`, beside the headline; 0 or 1: skip)")
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="also launch calibration_copy_kernel on a 256 MiB buffer this many times "
                          "(reference dispatches for scaling rocprofv3 byte counters)")
@@ -513,7 +573,8 @@ def main():
 
     # ---- the headline workload -------------------------------------------------------------------
     head, cases = measure_suite(torch, mk, args.suite, args.steps, args.warmup, yardstick, args.case_replays,
-                                with_dense=not args.no_dense, keep_dense=True)
+                                with_dense=not args.no_dense, keep_dense=True,
+                                concurrent_streams=args.overlap_streams)
     per_case = head["cases"]
 
     # ---- int8 values variant on the same sparsity patterns (densities 0.1 and 0.5 only) ------------
@@ -670,6 +731,7 @@ def main():
         "roofline": head["roofline"],
         "cpu_baseline": cpu,
         "streaming_read_yardstick": head.get("streaming_read_yardstick"),
+        "launches_overlapped": head.get("launches_overlapped"),
         "cases": per_case,
         "suites": suites,
         "compress": compress_cases,

@@ -75,6 +75,31 @@ def _decode_rope_attention_fake(q, k, v, cos_table, sin_table, position, k_cache
     return torch.empty_like(q)
 
 
+@torch.library.register_fake("macko_spmv::decode_rmsnorm")
+def _decode_rmsnorm_fake(x, weight, eps):
+    return torch.empty_like(x)
+
+
+@torch.library.register_fake("macko_spmv::decode_rope_append")
+def _decode_rope_append_fake(q, k, v, cos_table, sin_table, position, k_cache, v_cache):
+    return torch.empty_like(q)
+
+
+@torch.library.register_fake("macko_spmv::decode_attention")
+def _decode_attention_fake(q, k_cache, v_cache, position, scale):
+    return torch.empty_like(q)
+
+
+@torch.library.register_fake("macko_spmv::decode_silu_mul")
+def _decode_silu_mul_fake(gate, up):
+    return torch.empty_like(gate)
+
+
+# compress and compress_int8 have no fake implementation on purpose: the length of their outputs
+# depends on the data and the call waits for the GPU in the middle, so they run eagerly only
+# (torch.compile breaks the graph around them).
+
+
 @torch.library.register_fake("macko_spmv::multiply_int8")
 def _multiply_int8_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
     return torch.empty((M_rows,), device=V.device, dtype=V.dtype)

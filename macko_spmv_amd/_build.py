@@ -8,7 +8,7 @@ Both are built in-tree (next to this file) unless MACKO_SPMV_BUILD_DIRECTORY nam
 directory -- the same variable the upstream package reads for its JIT cache
 (src/macko_spmv/__init__.py:12).  hipcc cross-compiles for gfx950 without a GPU present.
 
-Run `python macko_spmv_amd/_build.py` to (re)build both.
+Run `python -m macko_spmv_amd._build` to (re)build them (`--devtools`: the tracing build and phase_trace).
 """
 import os
 import re

@@ -180,3 +180,21 @@ def test_assembly_check_of_the_hand_tracked_loads():
     with pytest.raises(RuntimeError, match="in front of a ring take"):
         _build.check_stream_kernel_assembly(
             head2 + [".LBB0_1:", "\ts_waitcnt vmcnt(0)", "\tv_or_b32_e32 v4, s2, v8"] + take2 + tail, name, base, slots)
+
+
+def test_build_directory_variable_redirects_every_artefact(tmp_path, monkeypatch):
+    """MACKO_SPMV_BUILD_DIRECTORY (upstream reads the same variable, src/macko_spmv/__init__.py:12)
+    moves the libraries, the benchmark library and the build stamp; nothing is current there
+    until something has been built there."""
+    from macko_spmv_amd import _build
+
+    in_tree = os.path.dirname(_build.lib_paths()[0])
+    target = tmp_path / "elsewhere"
+    monkeypatch.setenv("MACKO_SPMV_BUILD_DIRECTORY", str(target))
+    paths = [*_build.lib_paths(), _build.bench_lib_path(), _build.stamp_path()]
+    assert target.is_dir()
+    assert all(os.path.dirname(p) == str(target) for p in paths)
+    assert not _build.is_current()
+    monkeypatch.delenv("MACKO_SPMV_BUILD_DIRECTORY")
+    assert os.path.dirname(_build.lib_paths()[0]) == in_tree
+    assert _build.is_current()

@@ -187,6 +187,28 @@ def test_glue_kernels_match_torch_fp32():
 
 
 @pytest.mark.gpu
+def test_glue_kernels_have_fake_implementations():
+    """The unfused decode step can be traced: every glue operator passes opcheck (schema, fake
+    implementation against the real one, mutation annotations)."""
+    ops = torch.ops.macko_spmv
+    torch.manual_seed(4)
+    n_heads, head_dim, max_len, pos = 4, 64, 48, 5
+    H = n_heads * head_dim
+    x, w = torch.randn(H, device="cuda").half(), torch.ones(H, device="cuda").half()
+    q, k, v = (torch.randn(H, device="cuda").half() for _ in range(3))
+    inv = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda").float() / head_dim))
+    ang = torch.outer(torch.arange(max_len, device="cuda").float(), inv)
+    cos, sin = ang.cos().contiguous(), ang.sin().contiguous()
+    kc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+    vc = torch.randn(n_heads, max_len, head_dim, device="cuda").half()
+    position = torch.tensor([pos], device="cuda")
+    torch.library.opcheck(ops.decode_rmsnorm, (x, w, 1e-5))
+    torch.library.opcheck(ops.decode_silu_mul, (q, k))
+    torch.library.opcheck(ops.decode_rope_append, (q, k, v, cos, sin, position, kc, vc))
+    torch.library.opcheck(ops.decode_attention, (q, kc, vc, position, head_dim ** -0.5))
+
+
+@pytest.mark.gpu
 def test_concat_compressed_equals_compressing_the_stack():
     torch.manual_seed(5)
     mats = []
