@@ -232,3 +232,28 @@ def test_large_configuration_round_trip_and_product(rows, cols, density):
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.equal(out[:rows].float(), y) and float(out[rows]) == 7.0
+
+
+# ---- a malformed matrix: entries that decode to columns beyond `cols` --------------------------------
+
+@pytest.mark.parametrize("rows,wide,cols", [(300, 900, 600), (64, 40000, 30000)])
+def test_columns_beyond_cols_leave_the_other_rows_alone(rows, wide, cols):
+    """A well-formed matrix never decodes a column >= cols.  For one that does, upstream clamps the
+    column to cols - 1 (kernels.cuh:104-105); here the product of such a row is unspecified, but
+    the call must return normally and every row whose entries all lie inside `cols` must be right.
+    Built by compressing a wider matrix and passing a smaller column count."""
+    rng = np.random.default_rng(rows + cols)
+    dense = helpers.random_sparse(rng, rows, wide, 0.2)
+    dense[::3, cols:] = 0  # every third row stays inside `cols`
+    c = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    x = rng.standard_normal(cols).astype(np.float16)
+    print("case malformed", rows, wide, cols, flush=True)
+    y = macko_spmv.multiply((c[0], c[1], c[2], rows, cols), torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    y = y.cpu().numpy()
+    want = helpers.dense_reference(dense[::3, :cols], x)
+    helpers.assert_close_fp16(y[::3], want)
+    # the next call on the same stream is unaffected
+    good = macko_spmv.compress(torch.from_numpy(np.ascontiguousarray(dense[:, :cols])).cuda())
+    y2 = macko_spmv.multiply(good, torch.from_numpy(x).cuda()).cpu().numpy()
+    helpers.assert_close_fp16(y2, helpers.dense_reference(dense[:, :cols], x))
