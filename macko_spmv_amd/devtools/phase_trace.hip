@@ -9,6 +9,7 @@
 //
 // usage (from the repository root, or with MACKO_TRACE_LIBRARY naming the tracing library):
 //   phase_trace ROWS COLS DENSITY [ring-depth workgroups unused split(1|-1)]
+//   (a negative DENSITY gives rows of power-law length with mean -DENSITY)
 // build: python -m macko_spmv_amd._build --devtools
 #include <hip/hip_runtime.h>
 #include <dlfcn.h>
@@ -18,6 +19,7 @@
 #include <string.h>
 #include <vector>
 #include <algorithm>
+#include <cmath>
 #define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); exit(1);} } while (0)
 typedef int (*spmv_fn)(const void*, const void*, const int32_t*, const void*, void*, int32_t, int32_t, int64_t, void*);
 typedef int (*count_fn)(const void*, int32_t, int32_t, int32_t*, void*);
@@ -25,12 +27,14 @@ typedef int (*fill_fn)(const void*, int32_t, int32_t, const int32_t*, void*, voi
 typedef void (*tune_fn)(int, int, int, int);
 typedef void (*trace_fn)(long long*);
 __device__ inline uint32_t hash32(uint32_t x) { x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16; return x; }
-__global__ void k_gen_dense(uint16_t* M, int rows, int cols, float density, uint32_t seed)
+// row_density == nullptr: every element is kept with probability `density`; else row r with row_density[r]
+__global__ void k_gen_dense(uint16_t* M, int rows, int cols, float density, const float* row_density, uint32_t seed)
 {
     size_t n = (size_t)rows * cols;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         uint32_t h = hash32(hash32((uint32_t)i) ^ (seed * 0x9e3779b9u + 77u));
         float u = (h >> 8) * (1.0f / 16777216.0f);
+        if (row_density) density = row_density[i / cols];
         uint16_t v = 0;
         if (u < density) { v = (uint16_t)(0x2000 + (hash32(h) & 0x0fff)); if (h & 1) v |= 0x8000; }
         M[i] = v;
@@ -48,8 +52,24 @@ int main(int argc, char** argv)
     tune(argc > 4 ? atoi(argv[4]) : 0, argc > 5 ? atoi(argv[5]) : 0, argc > 6 ? atoi(argv[6]) : 0, argc > 7 ? atoi(argv[7]) : 0);
     hipStream_t s; CK(hipStreamCreate(&s));
     uint16_t* M; CK(hipMalloc(&M, (size_t)R * C * 2));
-    hipLaunchKernelGGL(k_gen_dense, dim3(2048), dim3(256), 0, s, M, R, C, d, 12345u);
-    int ncopy = (int)std::max<size_t>(3, std::min<size_t>(24, (size_t)1500000000 / ((size_t)R * C * d * 3 + 1)));
+    float* row_density = nullptr;
+    if (d < 0) {  // skewed rows: density ~ 0.01 * Pareto(1.5), clipped to [0.01, 0.95], rescaled to mean -d
+        std::vector<double> rd(R);
+        for (int r = 0; r < R; r++) {
+            uint32_t h = 0x9e3779b9u * (uint32_t)(r + 1); h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+            double u = ((h >> 8) + 0.5) / 16777216.0;
+            rd[r] = std::min(0.95, std::max(0.01, 0.01 * pow(1.0 - u, -1.0 / 1.5)));
+        }
+        for (int it = 0; it < 20; it++) {
+            double m = 0; for (double v : rd) m += v; m /= R;
+            for (double& v : rd) v = std::min(0.95, std::max(0.01, v * (-d / m)));
+        }
+        std::vector<float> rf(rd.begin(), rd.end());
+        CK(hipMalloc(&row_density, R * sizeof(float)));
+        CK(hipMemcpy(row_density, rf.data(), R * sizeof(float), hipMemcpyHostToDevice));
+    }
+    hipLaunchKernelGGL(k_gen_dense, dim3(2048), dim3(256), 0, s, M, R, C, d, row_density, 12345u);
+    int ncopy = (int)std::max<size_t>(3, std::min<size_t>(24, (size_t)1500000000 / ((size_t)((double)R * C * fabs(d) * 3) + 1)));
     std::vector<int*> rp(ncopy); std::vector<uint8_t*> v(ncopy), dl(ncopy);
     CK(hipMalloc(&rp[0], (R + 1) * 4));
     cnt(M, R, C, rp[0], s);
