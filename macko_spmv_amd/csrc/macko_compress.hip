@@ -518,8 +518,9 @@ int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_p
     if (rows < 0 || cols < 0 || row_ptr == nullptr) return MACKO_E_INVALID_ARGUMENT;
     if ((long long)rows * (long long)cols >= (1ll << 31)) return MACKO_E_INVALID_ARGUMENT;
     if (rows > 0 && cols > 0 && dense == nullptr) return MACKO_E_INVALID_ARGUMENT;
-    if ((reinterpret_cast<uintptr_t>(dense) & (sizeof(Elem) - 1)) || (reinterpret_cast<uintptr_t>(row_ptr) & 3))
-        return MACKO_E_INVALID_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(dense) & (sizeof(Elem) - 1)) || (reinterpret_cast<uintptr_t>(row_ptr) & 3) ||
+        (reinterpret_cast<uintptr_t>(total) & 3))
+        return MACKO_E_INVALID_ARGUMENT;  // before anything is launched
     hipStream_t s = as_stream(stream);
     if (rows > 0) {
         const bool stream_reads = streams_past_cache<Elem>(rows, cols);
@@ -533,7 +534,6 @@ int compress_count(const void *dense, int32_t rows, int32_t cols, int32_t *row_p
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
-    if (reinterpret_cast<uintptr_t>(total) & 3) return MACKO_E_INVALID_ARGUMENT;
     hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, s, row_ptr, rows, total);
     return (int)hipGetLastError();
 }

@@ -108,6 +108,16 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor, int64_t, int64_t> compress_on_dev
     const int64_t rows = M.size(0), cols = M.size(1);
     TORCH_CHECK(rows * cols < (1ll << 31), "matrix too large: rows * cols must stay below 2^31");
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    {
+        // The host has to wait for the entry count in the middle of this call, which a stream
+        // that is being captured into a graph cannot give: say so instead of breaking the capture.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        const hipError_t e = hipStreamIsCapturing(stream, &capturing);
+        TORCH_CHECK(e == hipSuccess, "macko_spmv: compress: ", hipGetErrorString(e));
+        TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
+                    "macko_spmv: compress cannot be captured into a HIP graph (the sizes of its outputs depend on "
+                    "the data); compress outside the capture and capture multiply only");
+    }
     const bool int8 = M.dtype() == at::kChar;
     at::Tensor row_ptr = at::empty({rows + 1}, M.options().dtype(at::kInt));
     // The entry count sizes the outputs, so the host has to wait for it.  The count pass stores it

@@ -495,45 +495,59 @@ def main(argv=None):
     ap.add_argument("--no-fuse", action="store_true",
                     help="engine path: keep rotary, the RMS norms and the SiLU gate as launches of their own")
     args = ap.parse_args(argv)
+    result = measure(density=args.density, layers=args.layers, dim=args.dim, hidden=args.hidden, heads=args.heads,
+                     vocab=args.vocab, prompt=args.prompt, tokens=args.tokens, runs=args.runs,
+                     skip_dense=args.skip_dense, module_path=args.module_path, compressed_file=args.compressed_file,
+                     fuse=not args.no_fuse)
+    print(json.dumps(result), flush=True)
+
+
+def measure(density=0.5, layers=32, dim=4096, hidden=11008, heads=32, vocab=32000, prompt=128, tokens=256, runs=3,
+            skip_dense=False, module_path=False, compressed_file=None, fuse=True):
+    """Builds the random-init model (dense, then with MACKO projections pruned to `density`), decodes
+    `tokens` tokens greedily behind a `prompt`-token prompt and returns tokens/s and memory figures
+    (the measurement of python_scripts/util_run_pruned_llm.py:201-207 upstream)."""
     assert torch.cuda.is_available(), "needs a GPU"
     torch.set_grad_enabled(False)
-    max_len = args.prompt + args.tokens + 8
-    result = {"density": args.density, "layers": args.layers, "prompt": args.prompt, "tokens": args.tokens,
-              "path": "module" if args.module_path else "engine",
-              "fused": not (args.module_path or args.no_fuse)}
+    max_len = prompt + tokens + 8
+    torch.cuda.empty_cache()
+    held_before = torch.cuda.memory_allocated()  # what the caller keeps on the device is not the model's
+    result = {"density": density, "layers": layers, "prompt": prompt, "tokens": tokens,
+              "path": "module" if module_path else "engine",
+              "fused": not (module_path or not fuse)}
     for label, sparse in (("dense", False), ("macko", True)):
-        if label == "dense" and args.skip_dense:
+        if label == "dense" and skip_dense:
             continue
-        model, proj_bytes = build_model(args.density, args.layers, args.dim, args.hidden, args.heads, args.vocab,
-                                        max_len, sparse=sparse and not args.compressed_file)
-        if sparse and args.compressed_file:
-            save_compressed_state_dict(compress_state_dict(model.state_dict()), args.compressed_file)
-            load_compressed_linears(model, load_compressed_state_dict(args.compressed_file, device="cuda"))
+        model, proj_bytes = build_model(density, layers, dim, hidden, heads, vocab,
+                                        max_len, sparse=sparse and not compressed_file)
+        if sparse and compressed_file:
+            save_compressed_state_dict(compress_state_dict(model.state_dict()), compressed_file)
+            load_compressed_linears(model, load_compressed_state_dict(compressed_file, device="cuda"))
             proj_bytes = sum(m.weight_bytes() for m in model.modules() if isinstance(m, MackoLinear))
             torch.cuda.empty_cache()
         engine = None
-        if not args.module_path:
-            engine = DecodeEngine(model, fuse=not args.no_fuse)
+        if not module_path:
+            engine = DecodeEngine(model, fuse=fuse)
             proj_bytes = engine.weight_bytes()
             torch.cuda.empty_cache()
-        resident = torch.cuda.memory_allocated()
+        resident = torch.cuda.memory_allocated() - held_before
         torch.cuda.reset_peak_memory_stats()  # the peak below covers prefill + decode, not model construction
         g = torch.Generator(device="cuda")
         g.manual_seed(1)
-        prompt = torch.randint(0, args.vocab, (1, args.prompt), device="cuda", generator=g)
+        prompt_ids = torch.randint(0, vocab, (1, prompt), device="cuda", generator=g)
         times = []
-        for _ in range(args.runs):
+        for _ in range(runs):
             if engine is not None:
-                ids, seconds = engine_decode(engine, prompt, args.tokens)
+                ids, seconds = engine_decode(engine, prompt_ids, tokens)
             else:
-                ids, seconds = greedy_decode(model, prompt, args.tokens)
+                ids, seconds = greedy_decode(model, prompt_ids, tokens)
             times.append(seconds)
         best = min(times)
         result[label] = {
-            "tokens_per_s": round((args.tokens - 1) / best, 2),
+            "tokens_per_s": round((tokens - 1) / best, 2),
             "projection_weights_gb": round(proj_bytes / 1e9, 3),
             "model_memory_gb": round(resident / 1e9, 3),
-            "peak_memory_gb": round(torch.cuda.max_memory_allocated() / 1e9, 3),
+            "peak_memory_gb": round((torch.cuda.max_memory_allocated() - held_before) / 1e9, 3),
             "first_tokens": ids[:8].tolist(),
         }
         print(label, result[label], file=sys.stderr, flush=True)
@@ -541,7 +555,7 @@ def main(argv=None):
         torch.cuda.empty_cache()
     if "dense" in result and "macko" in result:
         result["speedup"] = round(result["macko"]["tokens_per_s"] / result["dense"]["tokens_per_s"], 3)
-    print(json.dumps(result), flush=True)
+    return result
 
 
 if __name__ == "__main__":

@@ -87,6 +87,29 @@ def compress(dense_bits):
     return values[:p].copy(), deltas[: p // 2].copy(), row_ptr2, int(n)
 
 
+def compress_one_walk(dense_bits):
+    """The compressor as the upstream launcher runs it (cpu_compressor_torch_launcher.cuh:6-39): outputs
+    sized for the worst case (rows * cols entries), one walk over the matrix.  Returns
+    (values, deltas, row_ptr, n, seconds spent inside the C function)."""
+    import time
+
+    lib = _load()
+    dense_bits = _u16(dense_bits)
+    rows, cols = dense_bits.shape
+    cap = rows * cols + 8
+    values = np.zeros(cap, dtype=np.uint16)
+    deltas = np.zeros(cap // 2, dtype=np.uint8)
+    row_ptr = np.zeros(rows + 1, dtype=np.int32)
+    padded = ctypes.c_int64(0)
+    t0 = time.perf_counter()
+    n = lib.macko_oracle_compress_f16(_p(dense_bits), rows, cols, _p(row_ptr), _p(values), _p(deltas), cap,
+                                      ctypes.byref(padded))
+    seconds = time.perf_counter() - t0
+    assert n >= 0
+    p = padded.value
+    return values[:p].copy(), deltas[: p // 2].copy(), row_ptr, int(n), seconds
+
+
 def decode(values, deltas, row_ptr, rows, cols):
     lib = _load()
     values = _u16(values)

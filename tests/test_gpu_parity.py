@@ -430,3 +430,76 @@ def test_vmap_over_the_vector_like_the_upstream_llm_layer():
     out = lifted(x)
     assert out.shape == (6, 300)
     assert torch.allclose(out.float(), x[0].float() @ M.float().t(), rtol=1e-2, atol=2e-2)
+
+
+# ---- the upstream flow: compress on the host tensor, move the tuple, multiply ----------------------
+
+@pytest.mark.parametrize("shape,density", [((257, 1500), 0.3), ((64, 4096), 0.5), ((1000, 333), 0.05)])
+def test_cpu_compress_move_to_device_multiply(shape, density):
+    # src/macko_spmv/__init__.py:110-117 (move_to_device) between :120-131 (compress of a CPU tensor)
+    # and :134-149 (multiply): the route an upstream user takes when the dense matrix lives on the host
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    dense = helpers.random_sparse(rng, shape[0], shape[1], density)
+    dense[3] = 0
+    x = rng.standard_normal(shape[1]).astype(np.float16)
+    c_cpu = macko_spmv.compress(torch.from_numpy(dense))
+    assert all(t.device.type == "cpu" for t in c_cpu[:3])
+    _assert_bit_exact(c_cpu, dense)
+    c_gpu = macko_spmv.move_to_device(c_cpu, "cuda")
+    assert all(t.is_cuda for t in c_gpu[:3]) and c_gpu[3:] == c_cpu[3:]
+    # the moved tuple is what compress() gives for the same matrix on the GPU, bit for bit
+    direct = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    for moved, made in zip(c_gpu[:3], direct[:3]):
+        assert moved.dtype == made.dtype and torch.equal(moved, made)
+    y = macko_spmv.multiply(c_gpu, torch.from_numpy(x).cuda()).cpu().numpy()
+    values, deltas, row_ptr, _ = mo.compress(dense)
+    want = mo.spmv(values, deltas, row_ptr, shape[0], shape[1], x).view(np.float16)
+    assert np.allclose(y.astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=1e-3)
+    helpers.assert_close_fp16(y, helpers.dense_reference(dense, x))
+    # and back: nothing changes on the way
+    back = macko_spmv.move_to_device(c_gpu, "cpu")
+    for a, b in zip(back[:3], c_cpu[:3]):
+        assert a.device.type == "cpu" and torch.equal(a, b)
+    assert back[3:] == c_cpu[3:]
+
+
+def test_upstream_binding_names():
+    # the two pybind modules of the upstream package as attributes of the module
+    # (src/macko_spmv/__init__.py:36 `__compressor_lib`, :90 `__multiply_lib`, used at :124 and :141)
+    rng = np.random.default_rng(5)
+    dense = helpers.random_sparse(rng, 48, 700, 0.25)
+    x = torch.from_numpy(rng.standard_normal(700).astype(np.float16)).cuda()
+    compressor = getattr(macko_spmv, "__compressor_lib")
+    multiplier = getattr(macko_spmv, "__multiply_lib")
+    c = compressor.cpu_compress(torch.from_numpy(dense).cuda())
+    assert len(c) == 5 and c[3] == 48 and c[4] == 700
+    _assert_bit_exact(c, dense)
+    y = multiplier.macko_spmv_launcher(c[0], c[1], c[2], c[3], c[4], x)
+    assert y.dtype == torch.float16 and y.shape == (48,)
+    assert torch.equal(y, macko_spmv.multiply(c, x))
+    helpers.assert_close_fp16(y.cpu().numpy(), helpers.dense_reference(dense, x.cpu().numpy()))
+
+
+def test_compress_refuses_graph_capture():
+    # compress() has to read the entry count back in the middle of the call; under stream capture it
+    # says so, the capture survives, and a product captured next to it still replays correctly
+    rng = np.random.default_rng(11)
+    dense = helpers.random_sparse(rng, 96, 640, 0.3)
+    M = torch.from_numpy(dense).cuda()
+    x = torch.from_numpy(rng.standard_normal(640).astype(np.float16)).cuda()
+    c = macko_spmv.compress(M)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        y_eager = macko_spmv.multiply(c, x)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            with pytest.raises(RuntimeError, match="cannot be captured"):
+                macko_spmv.compress(M)
+            y_graph = macko_spmv.multiply(c, x)
+        for _ in range(3):
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(y_graph, y_eager)
+    torch.cuda.current_stream().wait_stream(stream)
