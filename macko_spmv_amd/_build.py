@@ -125,13 +125,15 @@ def check_stream_kernel_assembly(text, kernel_name="spmv_stream_kernel", fixed_b
     return checked
 
 
-def verify_fixed_registers(verbose=False):
-    """Compile the SpMV sources to assembly and run check_stream_kernel_assembly on each."""
+def verify_fixed_registers(verbose=False, extra_flags=()):
+    """Compile the SpMV sources to assembly (with `extra_flags`, so that a build with other
+    preprocessor settings is checked as it is built) and run check_stream_kernel_assembly on each."""
     checked = 0
     with tempfile.TemporaryDirectory() as tmp:
         for source, (kernel_name, fixed_base, slot_registers) in TRACKED_KERNELS.items():
             asm = os.path.join(tmp, source + ".s")
-            _run([_hipcc(), *_DEVICE_FLAGS, "--cuda-device-only", "-S", os.path.join(_CSRC, source), "-o", asm], verbose)
+            _run([_hipcc(), *_DEVICE_FLAGS, *extra_flags, "--cuda-device-only", "-S", os.path.join(_CSRC, source),
+                  "-o", asm], verbose)
             with open(asm) as f:
                 checked += check_stream_kernel_assembly(f.read().splitlines(), kernel_name, fixed_base, slot_registers)
     return checked
@@ -234,6 +236,7 @@ def build_devtools(verbose=False):
     here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "devtools")
     lib = os.path.join(here, "libmacko_hip_trace.so")
     tool = os.path.join(here, "phase_trace")
+    verify_fixed_registers(verbose, extra_flags=("-DMACKO_DEV_HOOKS",))  # the stamps are code between the takes
     _run([_hipcc(), *_DEVICE_FLAGS, "-DMACKO_DEV_HOOKS", "-fPIC", "-shared",
           *[os.path.join(_CSRC, s) for s in HIP_SOURCES], "-o", lib], verbose)
     _run([_hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", os.path.join(here, "phase_trace.hip"),

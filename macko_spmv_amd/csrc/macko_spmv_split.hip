@@ -18,67 +18,30 @@
 
 #include <atomic>
 
-#include "macko_spmv_detail.h"
+#include "macko_spmv_tracked.h"
 
 namespace macko {
 namespace {
 
 using namespace spmv_detail;
 
-// ---- loads whose completion is tracked by hand ---------------------------------------------
-// The tile ring, the row_ptr probes and the first pieces of x are fetched with inline-asm buffer
-// loads into FIXED physical VGPRs and awaited with explicit s_waitcnt vmcnt(N).  Vector-memory
-// loads complete in issue order, so "at most N loads outstanding" proves that every load older
-// than the N youngest has landed; N is always the number of tracked loads issued after the one
-// being awaited (loads or stores the compiler issues on its own can only make such a wait
-// longer, never too short).  The kernel is compiled with amdgpu_num_vgpr(kCompilerVgprs), which
-// keeps the register allocator below the fixed registers, so nothing else ever lives in them;
-// a `take` copies a landed slot into ordinary registers after its wait.  The byte offset goes
-// into the VGPR operand because only that operand takes part in the buffer's bounds check:
-// past-the-end addresses read as zero without touching memory, which is also how "no tile" is
-// encoded (kNoTile*).
-//
-// Register map (kCompilerVgprs = 84):  v84,v85 row_ptr probes; v86..v93 two 16-byte pieces of x;
-// v94..v103 ring (D <= 2): slot j keeps its values in v[94+4j : 97+4j] and its delta word in v[94+4D+j];
+// The hand-tracked loads (macko_spmv_tracked.h) with this kernel's register map: the compiler keeps
+// below v84; v84,v85 row_ptr probes; v86..v93 two 16-byte pieces of x; v94..v103 the ring (D <= 2);
 // v104..v119 four 16-byte pieces of the deltas in front of a wave's first entry ("look-back").
-
 constexpr int kCompilerVgprs = 84;
-#define MACKO_FIXED_CLOBBERS "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119"
-
-// row_ptr probe k (k = 0, 1) -> v84 + k
-template <int K>
-__device__ __forceinline__ void probe_issue(u32 byte_offset, const u32x4 &buffer)
+#define MACKO_SPLIT_FIXED_REGISTERS "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119"
+typedef TrackedLoads<kCompilerVgprs> Tracked;
+template <int K> __device__ __forceinline__ void probe_issue(u32 o, const u32x4 &b) { Tracked::probe_issue<K>(o, b); }
+template <int K, int N> __device__ __forceinline__ int probe_take() { return Tracked::probe_take<K, N>(); }
+template <int J> __device__ __forceinline__ void xpiece_issue(u32 o, const u32x4 &b) { Tracked::xpiece_issue<J>(o, b); }
+template <int J, int N> __device__ __forceinline__ void xpiece_to_lds(u32 a) { Tracked::xpiece_to_lds<J, N>(a); }
+template <int D, int J, int VB>
+__device__ __forceinline__ void ring_issue(u32 vo, u32 dof, const u32x4 &bv, const u32x4 &bd, bool stream)
 {
-    if (K == 0) asm volatile("buffer_load_dword v84, %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer) : "memory", "v84");
-    if (K == 1) asm volatile("buffer_load_dword v85, %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer) : "memory", "v85");
+    static_assert(D == 1 || D == 2, "ring depth");
+    Tracked::ring_issue<D, J, VB>(vo, dof, bv, bd, stream);
 }
-template <int K, int N>
-__device__ __forceinline__ int probe_take()
-{
-    int w;
-    if (K == 0) asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, v84" : "=v"(w) : "n"(N) : "memory");
-    if (K == 1) asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, v85" : "=v"(w) : "n"(N) : "memory");
-    return w;
-}
-
-// piece j of x (j = 0, 1) -> v[86+4j : 89+4j]
-template <int J>
-__device__ __forceinline__ void xpiece_issue(u32 byte_offset, const u32x4 &buffer)
-{
-    if (J == 0)
-        asm volatile("buffer_load_dwordx4 v[86:89], %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer)
-                     : "memory", "v86", "v87", "v88", "v89");
-    if (J == 1)
-        asm volatile("buffer_load_dwordx4 v[90:93], %0, %1, 0 offen" ::"v"(byte_offset), "s"(buffer)
-                     : "memory", "v90", "v91", "v92", "v93");
-}
-// waits for piece j and writes it to LDS straight from its registers
-template <int J, int N>
-__device__ __forceinline__ void xpiece_to_lds(u32 lds_byte_address)
-{
-    if (J == 0) asm volatile("s_waitcnt vmcnt(%1)\n\tds_write_b128 %0, v[86:89]" ::"v"(lds_byte_address), "n"(N) : "memory");
-    if (J == 1) asm volatile("s_waitcnt vmcnt(%1)\n\tds_write_b128 %0, v[90:93]" ::"v"(lds_byte_address), "n"(N) : "memory");
-}
+template <int D, int J, int N> __device__ __forceinline__ void ring_take(u32x4 &v, u32 &d) { Tracked::ring_take<D, J, N>(v, d); }
 
 // look-back piece j (j = 0..3) -> v[104+4j : 107+4j]
 template <int J>
@@ -104,59 +67,6 @@ __device__ __forceinline__ u32x4 look_take()
     return v;
 }
 
-// ring slot J of a D-deep ring: issue both loads / wait and copy out.  HINT is "" or " nt": the
-// matrix is read once per product, and a streaming read of that kind measures 11% faster with the
-// non-temporal hint at a few hundred MB.  The tiles a workgroup shares with its neighbours (its
-// first and last) go without it, so the second reader still finds them in L2.
-#define MACKO_RING_ISSUE(VREGS, DREG, HINT, CLOBBERS)                                                       \
-    asm volatile("buffer_load_dwordx4 " VREGS ", %0, %2, 0 offen" HINT "\n\tbuffer_load_dword " DREG         \
-                 ", %1, %3, 0 offen" HINT                                                                   \
-                 ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
-                 : "memory", CLOBBERS)
-#define MACKO_RING_TAKE(A, B, C, E, DREG)                                                                      \
-    asm volatile("s_waitcnt vmcnt(%5)\n\tv_mov_b32 %0, " A "\n\tv_mov_b32 %1, " B "\n\tv_mov_b32 %2, " C          \
-                 "\n\tv_mov_b32 %3, " E "\n\tv_mov_b32 %4, " DREG                                               \
-                 : "=v"(v.x), "=v"(v.y), "=v"(v.z), "=v"(v.w), "=v"(d) : "n"(N) : "memory")
-
-#define MACKO_RING_ISSUE_I8(VREGS, DREG, HINT, CLOBBERS)                                                    \
-    asm volatile("buffer_load_dwordx2 " VREGS ", %0, %2, 0 offen" HINT "\n\tbuffer_load_dword " DREG         \
-                 ", %1, %3, 0 offen" HINT                                                                   \
-                 ::"v"(values_offset), "v"(deltas_offset), "s"(buf_values), "s"(buf_deltas)                  \
-                 : "memory", CLOBBERS)
-// `stream` is wave-uniform
-#define MACKO_RING_ISSUE_EITHER(MACRO, VREGS, DREG)                \
-    do {                                                           \
-        if (stream)                                                \
-            MACRO(VREGS, DREG, " nt", MACKO_FIXED_CLOBBERS);       \
-        else                                                       \
-            MACRO(VREGS, DREG, "", MACKO_FIXED_CLOBBERS);          \
-    } while (0)
-
-// VB = bytes per stored value: 2 (fp16, 16 bytes per lane and tile) or 1 (int8, 8 bytes per lane
-// and tile, which land in the first two registers of the slot).
-template <int D, int J, int VB>
-__device__ __forceinline__ void ring_issue(u32 values_offset, u32 deltas_offset, const u32x4 &buf_values,
-                                           const u32x4 &buf_deltas, bool stream)
-{
-    static_assert(D == 1 || D == 2, "ring depth");
-    if (VB == 1) {
-        if (D == 1 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[94:95]", "v98");
-        if (D == 2 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[94:95]", "v102");
-        if (D == 2 && J == 1) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE_I8, "v[98:99]", "v103");
-        return;
-    }
-    if (D == 1 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[94:97]", "v98");
-    if (D == 2 && J == 0) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[94:97]", "v102");
-    if (D == 2 && J == 1) MACKO_RING_ISSUE_EITHER(MACKO_RING_ISSUE, "v[98:101]", "v103");
-}
-
-template <int D, int J, int N>
-__device__ __forceinline__ void ring_take(u32x4 &v, u32 &d)
-{
-    if (D == 1 && J == 0) MACKO_RING_TAKE("v94", "v95", "v96", "v97", "v98");
-    if (D == 2 && J == 0) MACKO_RING_TAKE("v94", "v95", "v96", "v97", "v102");
-    if (D == 2 && J == 1) MACKO_RING_TAKE("v98", "v99", "v100", "v101", "v103");
-}
 
 // NB = vectors multiplied per launch (1, 2, 4 or 8).  With NB > 1 the NB copies of x are interleaved in
 // LDS (element c of vector b at half-word c * NB + b), so one LDS read per stored entry fetches the
@@ -173,6 +83,7 @@ spmv_split_kernel(const SpmvArgs a)
     static_assert(NB == 1 || (NB <= 8 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
     static_assert(XF == 0 || (NB == 1 && X_LDS && VB == 2), "fused staging: fp16, one vector, x in LDS");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    MACKO_RESERVE_FIXED_REGISTERS(MACKO_SPLIT_FIXED_REGISTERS);
     constexpr int WAVES = BLOCK / kWave;
     constexpr int kBatchShift = NB == 8 ? 3 : (NB == 4 ? 2 : (NB == 2 ? 1 : 0));
     constexpr int kTileLoads = 2 * D;  // tracked loads per full ring
@@ -238,95 +149,7 @@ spmv_split_kernel(const SpmvArgs a)
     // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
     //         x, goes to LDS through ordinary loads (rare: more than 16384 columns, or an x that is
     //         not 16-byte aligned) ------------------------------------------------------------------
-    if (NB > 1) {
-        // every vector through ordinary loads, interleaved: element c of vector b at dst[c * NB + b]
-        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront * NB);
-        const bool vec_ok = x_vec && (a.ldx & 7) == 0;
-        const int nvec = vec_ok ? a.cols >> 3 : 0;
-        // 8 columns of every vector per thread and step: NB 16-byte loads, interleaved in registers,
-        // written back as NB 16-byte stores (16 * NB contiguous bytes of LDS)
-        for (int i = tid; i < nvec; i += BLOCK) {
-            u32x4 v[NB];
-#pragma unroll
-            for (int b = 0; b < NB; ++b)
-                v[b] = reinterpret_cast<const u32x4 *>(a.x + (size_t)b * (size_t)a.ldx)[i];
-            u32 out[4 * NB];  // half-word (c * NB + b) = element c of vector b
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-#pragma unroll
-                for (int b = 0; b < NB; b += 2) {
-                    const u32 lo = (v[b][c >> 1] >> (16 * (c & 1))) & 0xffffu;
-                    const u32 hi = (v[b + 1][c >> 1] >> (16 * (c & 1))) & 0xffffu;
-                    out[(c * NB + b) >> 1] = lo | (hi << 16);
-                }
-            }
-            u32x4 *d4 = reinterpret_cast<u32x4 *>(dst + (size_t)8 * i * NB);
-#pragma unroll
-            for (int q = 0; q < NB; ++q) d4[q] = u32x4{out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]};
-        }
-#pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            const uint16_t *xb = a.x + (size_t)b * (size_t)a.ldx;
-            for (int i = (nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i * NB + b] = xb[i];
-        }
-        if (tid < kLdsFront * NB / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-        if (tid < kLdsBack * NB / 2) dst[a.cols * NB + tid] = 0;
-    } else if (XF != 0) {
-        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
-        const int nvec = a.cols >> 3;
-        auto lo = [](u32 w) { return half_bits_to_float((uint16_t)(w & 0xffffu)); };
-        auto hi = [](u32 w) { return half_bits_to_float((uint16_t)(w >> 16)); };
-        auto pack = [](float l, float h) { return (u32)float_to_half_bits(l) | ((u32)float_to_half_bits(h) << 16); };
-        if (XF == 1) {
-            // pass 1: raw x into LDS and the sum of squares; pass 2: each thread scales the pieces
-            // it wrote itself, so only the sum needs a barrier
-            float ss = 0.f;
-            for (int i = tid; i < nvec; i += BLOCK) {
-                const u32x4 v = reinterpret_cast<const u32x4 *>(a.x)[i];
-                d4[i] = v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) ss += lo(v[e]) * lo(v[e]) + hi(v[e]) * hi(v[e]);
-            }
-            float *red = reinterpret_cast<float *>(lds + kLdsFront + 2 * (size_t)a.cols + kLdsBack);
-            const float ws = wave_sum(ss);
-            if (lane == 0) red[wave] = ws;
-            __syncthreads();
-            float total = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) total += red[w];
-            const float inv = rsqrtf(total / (float)a.cols + a.eps);
-            for (int i = tid; i < nvec; i += BLOCK) {
-                const u32x4 v = d4[i];
-                const u32x4 g = reinterpret_cast<const u32x4 *>(a.x2)[i];
-                u32x4 o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = pack(lo(v[e]) * inv * lo(g[e]), hi(v[e]) * inv * hi(g[e]));
-                d4[i] = o;
-            }
-        } else {
-            auto gate = [](float g, float u) { return g / (1.0f + __expf(-g)) * u; };
-            for (int i = tid; i < nvec; i += BLOCK) {
-                const u32x4 g = reinterpret_cast<const u32x4 *>(a.x)[i];
-                const u32x4 u = reinterpret_cast<const u32x4 *>(a.x2)[i];
-                u32x4 o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = pack(gate(lo(g[e]), lo(u[e])), gate(hi(g[e]), hi(u[e])));
-                d4[i] = o;
-            }
-        }
-        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
-    } else if (X_LDS) {
-        uint16_t *dst = reinterpret_cast<uint16_t *>(lds + kLdsFront);
-        u32x4 *d4 = reinterpret_cast<u32x4 *>(dst);
-        if (__builtin_expect(x_nvec > kXRegs * BLOCK, 0))
-            for (int i = tid + kXRegs * BLOCK; i < x_nvec; i += BLOCK) d4[i] = reinterpret_cast<const u32x4 *>(a.x)[i];
-        if (__builtin_expect((x_nvec << 3) < a.cols, 0))
-            for (int i = (x_nvec << 3) + tid; i < a.cols; i += BLOCK) dst[i] = a.x[i];
-        if (tid < kLdsFront / 4) reinterpret_cast<u32 *>(lds)[tid] = 0;
-        if (tid < kLdsBack / 2) dst[a.cols + tid] = 0;
-    }
+    stage_x_untracked<BLOCK, X_LDS, NB, XF>(lds, a, tid, lane, wave, x_vec, x_nvec);
     MACKO_STAMP(1);
 
     constexpr int kXLoads = X_LDS && NB == 1 && XF == 0 ? kXRegs : 0;
