@@ -167,8 +167,10 @@ spmv_stream_kernel(const SpmvArgs a)
         // Straight-line case: both cuts fall inside their probe windows and my first row is not
         // empty.  Cut k is the first row start at or after target k, or the one before it if that
         // is nearer (with rows of similar length every wave then gets the same number of rows).
-        const unsigned long long m0 = __ballot(window[0] >= target[0]);
-        const unsigned long long m1 = __ballot(window[1] >= target[1]);
+        // (cuts are taken on row_ptr[r] + row_cost * r: see SpmvArgs::row_cost)
+        const int row_cost = (int)a.row_cost;
+        const unsigned long long m0 = __ballot(window[0] + row_cost * (base[0] + lane) >= target[0]);
+        const unsigned long long m1 = __ballot(window[1] + row_cost * (base[1] + lane) >= target[1]);
         const int f0 = m0 ? __builtin_ctzll(m0) : 0;
         const int f1 = m1 ? __builtin_ctzll(m1) : 0;
         if (a.row_even) {  // the cuts are the guesses themselves; both lie inside their windows
@@ -186,8 +188,9 @@ spmv_stream_kernel(const SpmvArgs a)
             const int before0 = __builtin_amdgcn_readlane(window[0], f0 - 1);
             const int at1 = __builtin_amdgcn_readlane(window[1], f1);
             const int before1 = __builtin_amdgcn_readlane(window[1], f1 - 1);
-            const int back0 = target[0] - before0 < at0 - target[0] ? 1 : 0;
-            const int back1 = target[1] - before1 < at1 - target[1] ? 1 : 0;
+            const int weight0 = row_cost * (base[0] + f0), weight1 = row_cost * (base[1] + f1);
+            const int back0 = target[0] - (before0 + weight0 - row_cost) < at0 + weight0 - target[0] ? 1 : 0;
+            const int back1 = target[1] - (before1 + weight1 - row_cost) < at1 + weight1 - target[1] ? 1 : 0;
             r = base[0] + f0 - back0;
             row_last = base[1] + f1 - back1;
             e0 = back0 ? before0 : at0;
@@ -201,7 +204,8 @@ spmv_stream_kernel(const SpmvArgs a)
     if (__builtin_expect(!resolved, 0)) {
         // General case: search rounds where a window missed, first / last wave, leading empty rows.
         int range[2] = {guess[0], guess[1]};
-        if (!a.row_even) wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range);
+        const int row_cost = (int)a.row_cost;
+        if (!a.row_even) wave_lower_bound2(a.row_ptr, a.rows, lane, target, window, base, range, row_cost);
 #pragma unroll
         for (int k = 0; k < 2 && !a.row_even; ++k) {
             const int rr = range[k];
@@ -214,7 +218,7 @@ spmv_stream_kernel(const SpmvArgs a)
                     after = uniform(a.row_ptr[rr]);
                     before = uniform(a.row_ptr[rr - 1]);
                 }
-                if (target[k] - before < after - target[k]) range[k] = rr - 1;
+                if (target[k] - (before + row_cost * (rr - 1)) < after + row_cost * rr - target[k]) range[k] = rr - 1;
             }
         }
         if (gw == 0) range[0] = 0;
@@ -490,8 +494,14 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
     auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
-    a.entries_q = (u32)(a.padded / n_waves);
-    a.entries_rem = (u32)(a.padded % n_waves);
+    {
+        // the sum the waves share evenly: stored entries plus row_cost per row (kept below 2^31)
+        const long long room = ((1ll << 31) - 1 - a.padded) / (a.rows > 0 ? a.rows : 1);
+        if ((long long)a.row_cost > room) a.row_cost = (u32)room;
+        const long long weight = a.padded + (long long)a.row_cost * a.rows;
+        a.entries_q = (u32)(weight / n_waves);
+        a.entries_rem = (u32)(weight % n_waves);
+    }
     a.rows_q = (u32)a.rows / n_waves;
     a.rows_frac = (u32)(((unsigned long long)((u32)a.rows % n_waves) << 32) / n_waves);
     a.row_even = (u32)a.rows <= n_waves ? 1u : 0u;
@@ -512,12 +522,18 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
     return (int)hipGetLastError();
 }
 
+// What a row weighs, in entries, when rows are dealt to waves (SpmvArgs::row_cost): one tile.
+// Measured on 14336 x 4096 matrices whose row lengths follow a Pareto law (41 to 3900 entries a
+// row): 5 to 9 % faster than cuts on entries alone; matrices of equal rows do not change.
+constexpr u32 kRowCost = 512;
+
 #ifdef MACKO_DEV_HOOKS
 // Launch-shape overrides for tuning runs (0 = built-in default); development builds only.
 struct Tuning {
     int depth;  // tiles in flight per wave: 1 or 2
     int grid;   // workgroups
     int split;  // 1: always the split kernel, -1: never
+    int row_cost;  // what a row weighs in the cuts, in entries (-1: built-in)
 };
 Tuning g_tuning = {0, 0, 0};
 long long *g_trace = nullptr;
@@ -575,7 +591,9 @@ int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
     // start, when a wave walks only a few tiles; from about four tiles per wave on, two do better
     // (measured on the Llama shapes and larger ones, fp16 and int8; deeper is slower).
     int depth = n_tiles >= 4 * grid * waves ? 2 : 1;
+    a.row_cost = kRowCost;
 #ifdef MACKO_DEV_HOOKS
+    if (g_tuning.row_cost >= 0) a.row_cost = (u32)g_tuning.row_cost;
     if (g_tuning.depth) depth = g_tuning.depth;
     if (g_tuning.grid) grid = g_tuning.grid;
 #endif
@@ -622,8 +640,7 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 extern "C" void macko_spmv_set_trace(long long *device_buffer) { macko::g_trace = device_buffer; }
 extern "C" void macko_spmv_tune(int depth, int grid, int active, int split)
 {
-    (void)active;
-    macko::g_tuning = macko::Tuning{depth, grid, split};
+    macko::g_tuning = macko::Tuning{depth, grid, split, active > 0 ? active - 1 : -1};
 }
 #endif
 

@@ -48,6 +48,10 @@ struct SpmvArgs {
     // wave that starts inside a row at which column it continues): 512, or 2048 * k, k = 1..4.
     // Chosen from the mean row length; rows that began further back cost an extra round trip.
     u32 look_entries;
+    // Whole-row kernel only.  What a row weighs, in stored entries, when the rows are dealt to the
+    // waves: the cuts balance entries + row_cost * rows (a row's end costs a reduction, a store and
+    // masked passes, whatever its length).  entries_q / entries_rem then split that sum.
+    u32 row_cost;
 #ifdef MACKO_DEV_HOOKS
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif
@@ -97,16 +101,18 @@ __device__ __forceinline__ int load_row_window(const int *__restrict__ row_ptr, 
 // the ones just seen (which usually lands within a few rows even for very uneven matrices; that
 // window then replaces window[k] / base[k] so the caller finds its row starts in it), and 64-ary
 // rounds over what is still undecided follow.  Every value here is wave-uniform.
+// With row_cost != 0 the search runs on row_ptr[r] + row_cost * r instead of row_ptr[r] (a row then
+// weighs row_cost entries on top of its own); the windows keep plain row_ptr values.
 __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_ptr, int rows, int lane,
                                                   const int target[2], int (&window)[2], int (&base)[2],
-                                                  int out[2])
+                                                  int out[2], int row_cost = 0)
 {
     int lo[2], hi[2];
     // narrows [lo, hi] with a window of row_ptr values: probed[i] >= target puts the answer at or
     // before base + i, probed[i] < target puts it after
     auto narrow = [&](int k, int probed, int at) {
         const bool beyond = at + lane > rows;
-        const unsigned long long m = __ballot(beyond || probed >= target[k]);
+        const unsigned long long m = __ballot(beyond || probed + row_cost * (at + lane) >= target[k]);
         if (m == 0) {
             const int after = at + 64 > rows ? rows : at + 64;
             lo[k] = lo[k] > after ? lo[k] : after;
@@ -132,8 +138,8 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
             at[k] = base[k];
             if (lo[k] < hi[k]) {
                 const int last = base[k] + 63 <= rows ? 63 : rows - base[k];
-                const int v0 = __builtin_amdgcn_readlane(window[k], 0);
-                const int v1 = __builtin_amdgcn_readlane(window[k], last);
+                const int v0 = __builtin_amdgcn_readlane(window[k], 0) + row_cost * base[k];
+                const int v1 = __builtin_amdgcn_readlane(window[k], last) + row_cost * (base[k] + last);
                 const float per_entry = (float)(last > 0 ? last : 1) / (float)(v1 > v0 ? v1 - v0 : 1);
                 float jump = (float)(target[k] - v0) * per_entry;
                 jump = jump > 2.0e9f ? 2.0e9f : (jump < -2.0e9f ? -2.0e9f : jump);
@@ -161,7 +167,7 @@ __device__ __forceinline__ void wave_lower_bound2(const int *__restrict__ row_pt
         for (int k = 0; k < 2; ++k) {
             step[k] = (hi[k] - lo[k] + 63) >> 6;
             const int idx = lo[k] + lane * step[k];
-            probe[k] = (lo[k] < hi[k] && idx < hi[k]) ? row_ptr[idx] : 0x7fffffff;
+            probe[k] = (lo[k] < hi[k] && idx < hi[k]) ? row_ptr[idx] + row_cost * idx : 0x7fffffff;
         }
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
