@@ -85,7 +85,8 @@ def check_stream_kernel_assembly(text, kernel_name="spmv_stream_kernel", fixed_b
     blocks no instruction touches a VGPR >= fixed_base, and the compiler has put no vmcnt wait of its
     own right in front of a ring take (it does when one of its own loads may still be outstanding at
     the loop's back edge; such a wait also waits for the ring loads in flight and serialises the
-    stream).  Returns the number of kernels checked; raises RuntimeError on a violation."""
+    stream).  Also checks that no kernel of the file calls a function or uses scratch memory.
+    Returns the number of kernels checked; raises RuntimeError on a violation."""
     kernel = None
     in_asm = False
     checked = 0
@@ -122,6 +123,16 @@ def check_stream_kernel_assembly(text, kernel_name="spmv_stream_kernel", fixed_b
                 raise RuntimeError(f"compiler-generated code touches a fixed VGPR in {kernel}: {line.strip()}")
     if checked == 0:
         raise RuntimeError(f"no {kernel_name} found in the assembly; the register check is stale")
+    # No kernel of these files may call a function or keep anything in scratch memory: a lambda of
+    # the kernel that is not inlined takes its captures, the kernel's whole state, through memory
+    # (measured: four times slower), and its code would not be covered by the checks above.
+    for number, line in enumerate(text):
+        code = line.split(";")[0]
+        if re.search(r"\bs_swappc_b64\b|\bscratch_(load|store)_", code):
+            raise RuntimeError(f"function call or scratch access in the assembly (line {number + 1}): {code.strip()}")
+        m = re.search(r"\.amdhsa_private_segment_fixed_size\s+(\d+)", code)
+        if m and int(m.group(1)) != 0:
+            raise RuntimeError(f"a kernel uses {m.group(1)} bytes of scratch memory (assembly line {number + 1})")
     return checked
 
 

@@ -54,12 +54,17 @@ template <int D, int J, int N> __device__ __forceinline__ void ring_take(u32x4 &
 // launch of its own: 0 = none (x as given), 1 = RMS norm (x * rsqrt(mean(x^2) + eps) * x2, x2 the
 // norm weight), 2 = SiLU gate (silu(x) * x2).  The staged vector is rounded to fp16 exactly as a
 // separate kernel writing it to memory would.  XF != 0 needs cols % 8 == 0 and 16-byte aligned x, x2.
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB, int XF>
+// ROWS = with the pass that works all the rows of a tile at once (rows_pass below), for matrices of
+// short rows.  A variant of its own: compiled into the kernel, that pass costs the row loop of
+// every matrix 0.3 to 0.7 us per launch (measured on 4096 x 4096 and 11008 x 4096 at density 0.1),
+// used or not.
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB, int XF, bool ROWS>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
     static_assert(NB == 1 || (NB <= 8 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
     static_assert(XF == 0 || (NB == 1 && X_LDS && VB == 2), "fused staging: fp16, one vector, x in LDS");
+    static_assert(!ROWS || (X_LDS && NB == 1 && XF == 0), "all rows of a tile in one pass: one vector, x in LDS");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     MACKO_RESERVE_FIXED_REGISTERS(MACKO_STREAM_FIXED_REGISTERS);
     constexpr int WAVES = BLOCK / kWave;
@@ -313,7 +318,7 @@ spmv_stream_kernel(const SpmvArgs a)
     // their value is masked to zero, but what they would read lies behind the row's last column
     // and may be Inf or NaN, so they read the zero bytes in front of x instead.  (Entries in front
     // of kmin, masked at a row's start, read those zero bytes by construction when x is in LDS.)
-    auto lane_fma = [&](const u32x4 &vv, u32 dd, u32 base, auto checked, int kmin, int kmax) {
+    auto lane_fma = [&](const u32x4 &vv, u32 dd, u32 base, auto checked, int kmin, int kmax) __attribute__((always_inline)) {
         constexpr bool CHECKED = decltype(checked)::value != 0;
         const u32 zeros = row_origin - 16u;  // 16 zero bytes (times NB) in front of x
 #pragma unroll
@@ -371,7 +376,7 @@ spmv_stream_kernel(const SpmvArgs a)
     // A tile that lies wholly inside the current row: no masks, every lane active.  Each lane
     // advances the row address by 16 bytes (its 8 entries) plus twice its nibble sum; the DPP scan
     // of that quantity gives every lane its starting address.
-    auto full_tile_pass = [&](const u32x4 &vj, u32 dj) {
+    auto full_tile_pass = [&](const u32x4 &vj, u32 dj) __attribute__((always_inline)) {
         const u32 step = __builtin_amdgcn_udot8(dj, 0x22222222u, 16u, false);
         const u32 incl = (u32)wave_scan_inclusive((int)step);
         const u32 base = (incl - step) + row_addr;
@@ -382,7 +387,7 @@ spmv_stream_kernel(const SpmvArgs a)
     // Entries [pos, seg_end) of the tile starting at entry `tb`, all in the current row: lanes
     // outside the segment are switched off, the first and last lane of the segment are masked.
     // A row that starts `q0` entries into its first lane shifts every address by -2*q0.
-    auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end, auto checked) {
+    auto segment_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int seg_end, auto checked) __attribute__((always_inline)) {
         const int rel0 = pos - tb;
         const int rel1 = seg_end - tb;
         const int l0 = rel0 >> 3, q0 = rel0 & 7;
@@ -403,7 +408,7 @@ spmv_stream_kernel(const SpmvArgs a)
         if (active) lane_fma(vv, dd, base, checked, kmin, kmax);
     };
 
-    auto finish_row = [&](float total) {  // total: the row's sum where there is one vector
+    auto finish_row = [&](float total) __attribute__((always_inline)) {  // total: the row's sum where there is one vector
         if (NB == 1) {
             store_row(r, total);
             acc0 = acc1 = 0.f;
@@ -423,6 +428,131 @@ spmv_stream_kernel(const SpmvArgs a)
             e1 = row_start(r + 1);
             if (e1 == e0) store_empty_row(r);
         } while (e1 == e0);
+    };
+
+    // Entries [pos, stop) of the tile starting at entry `tb`, over all the rows they belong to at
+    // once: for tiles in which several rows end, where a pass per row (segment_pass) would cost a
+    // scan, eight multiply-adds, a reduction and a store per row, however short.  Here the column
+    // addresses and the sums are segmented prefix scans that restart where a row starts:
+    //   1. the rows of the window mark their first entry in a per-lane bit mask (through LDS);
+    //   2. every lane walks its 8 entries from the address the scan hands it, back to x[0] at a mark;
+    //   3. the products are summed the same way; every entry's running row sum goes to LDS;
+    //   4. the window's lanes, one per row, fetch the sum at their row's last entry and store y.
+    // `stop` is the tile's end, the end of my rows, or the start of the window's last row,
+    // whichever comes first; the current row r may have begun in an earlier tile (its partial sums
+    // are in acc0 / acc1, its address in row_addr).  Leaves r, e0, e1, acc0, acc1, row_addr as the
+    // row loop expects them at entry `stop`.  No entry is masked: every entry in [pos, stop) is
+    // read at its own column, and what lies outside never reaches a stored sum.
+    auto rows_pass = [&](const u32x4 &vj, u32 dj, int tb, int pos, int stop) __attribute__((always_inline)) {
+        typedef __attribute__((address_space(3))) u32 *lds_w32;
+        typedef __attribute__((address_space(3))) float *lds_f32;
+        typedef __attribute__((address_space(3))) u32x4 *lds_w32x4;
+        auto bits = [](float f) { return __builtin_bit_cast(u32, f); };
+        const u32 area = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + a.rows_pass_lds +
+                         (u32)wave * (kTile * 4);
+        const int rw_end = row_last < win_base + 63 ? row_last : win_base + 63;  // last row whose start I know
+        const int row_j = win_base + lane;
+        const int e_j = win;
+        const int e_next = wave_from_lane_above(win);
+        const bool continuing = e0 < tb;
+        const float carry_sum = continuing ? wave_sum(acc0 + acc1) : 0.f;
+        const u32 carry_addr = row_addr - row_origin;
+
+        // 1. marks
+        *(lds_w32)(uintptr_t)(area + lane4) = 0u;
+        __builtin_amdgcn_wave_barrier();
+        if (row_j >= r && row_j <= rw_end && e_j >= pos && e_j > tb && e_j <= stop && e_j < tb + kTile) {
+            const u32 rel = (u32)(e_j - tb);
+            __hip_atomic_fetch_or((lds_w32)(uintptr_t)(area + (rel >> 3) * 4), 1u << (rel & 7), __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+        __builtin_amdgcn_wave_barrier();
+        const u32 marks = *(lds_w32)(uintptr_t)(area + lane4);
+        const bool marked = marks != 0;
+        const SegmentMasks seg = segment_masks(__ballot(marked));
+
+        // 2. addresses: what a lane passes on is its walk from its last mark (all 8 entries if none)
+        const int last_mark = marked ? 31 - __builtin_clz(marks) : 0;
+        u32 walk = __builtin_amdgcn_udot8(dj & (~0u << (4 * last_mark)), 0x22222222u, 2u * (u32)(8 - last_mark), false);
+        if (lane == 0 && !marked) walk += carry_addr;
+        const u32 walk_incl = wave_segmented_scan<u32>(walk, seg);
+        u32 run = (u32)wave_from_lane_below((int)walk_incl);
+        if (lane == 0) run = carry_addr;
+        run += row_origin;
+        const int rel0 = pos - tb, rel1 = stop - tb;
+        const bool active = lane >= (rel0 >> 3) && lane <= ((rel1 - 1) >> 3);
+
+        // 3. products and running row sums
+        float t[8];
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const bool mark = (marks >> k) & 1u;
+            run = mark ? row_origin : run;
+            const u32 addr = run + 2u * ((dj >> (4 * k)) & 15u);
+            run = addr + 2u;
+            uint16_t xb = 0;
+            if (active) xb = *(lds_u16_ptr)(uintptr_t)addr;
+            float m;
+            if (VB == 2) {
+                const u32 w = vj[k >> 1];
+                m = half_bits_to_float((k & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+            } else {
+                m = (float)((int)(vj[k >> 2] << (24 - 8 * (k & 3))) >> 24);
+            }
+            sum = mark ? 0.f : sum;
+            sum = __builtin_fmaf(m, half_bits_to_float(xb), sum);
+            t[k] = sum;
+        }
+        const float sum_incl = wave_segmented_scan<float>(sum, seg);
+        const float before = __builtin_bit_cast(float, wave_from_lane_below(__builtin_bit_cast(int, sum_incl)));
+        *(lds_w32x4)(uintptr_t)(area + (u32)lane * 32) = u32x4{bits(t[0]), bits(t[1]), bits(t[2]), bits(t[3])};
+        *(lds_w32x4)(uintptr_t)(area + (u32)lane * 32 + 16) = u32x4{bits(t[4]), bits(t[5]), bits(t[6]), bits(t[7])};
+        __builtin_amdgcn_wave_barrier();
+        // the entries in front of a lane's first mark continue the row of the lanes before: only the
+        // last of them can end a row, so only its sum needs what those lanes add
+        if ((marks & 1u) == 0) {
+            const int fix = marked ? __builtin_ctz(marks) - 1 : 7;
+            __hip_atomic_fetch_add((lds_f32)(uintptr_t)(area + (u32)lane * 32 + (u32)fix * 4), before, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        // 4. one lane per row that ends in [pos, stop]
+        if (row_j >= r && row_j < rw_end && e_next <= stop) {
+            float total = 0.f;
+            if (e_next != e_j) {
+                total = *(lds_f32)(uintptr_t)(area + (u32)(e_next - 1 - tb) * 4);
+                if (row_j == r) total += carry_sum;
+            }
+            float out = total;
+            if (AXPBY) out = a.alpha * total + a.beta * half_bits_to_float(a.y[row_j]);
+            a.y[row_j] = float_to_half_bits(out);
+        }
+
+        // the row that holds entry `stop`
+        const unsigned long long begun = __ballot(row_j >= r && row_j <= rw_end && e_j <= stop);
+        const int open_row = r + __builtin_popcountll(begun) - 1;
+        float open_sum = 0.f;
+        u32 open_addr = row_origin;
+        if (stop == tb + kTile) {
+            open_sum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum_incl), kWave - 1));
+            if (open_row == r) open_sum += carry_sum;
+            open_addr = row_origin + (u32)__builtin_amdgcn_readlane((int)walk_incl, kWave - 1);
+        }
+        r = open_row - 1;
+        do {
+            ++r;
+            if (r >= row_last) break;
+            slide_window(r);
+            e0 = row_start(r);
+            e1 = row_start(r + 1);
+            if (e1 == e0) store_empty_row(r);
+        } while (e1 == e0);
+        const bool open = r < row_last && e0 < stop;
+        acc0 = (open && lane == 0) ? open_sum : 0.f;
+        acc1 = 0.f;
+        row_addr = open ? open_addr : row_origin;
     };
 
     // The ring holds my first D tiles; now: take a slot, refill it, process.  Every step issues
@@ -446,6 +576,18 @@ spmv_stream_kernel(const SpmvArgs a)
                 const int lim = tile_end < s_end ? tile_end : s_end;
                 int pos = tb > e0 ? tb : e0;  // e0 > tb only in my first tile
                 while (pos < lim) {
+                    if constexpr (ROWS) {
+                        // several rows end in what is left of this tile: all of them in one pass
+                        const int ahead = r + (int)a.rows_pass_min;
+                        if (ahead <= row_last && ahead <= win_base + 63 && row_start(ahead) <= lim) {
+                            const int known = row_last < win_base + 63 ? row_last : win_base + 63;
+                            const int known_start = row_start(known);
+                            const int stop = known_start < lim ? known_start : lim;
+                            rows_pass(vj, dj, tb, pos, stop);
+                            pos = stop;
+                            continue;
+                        }
+                    }
                     const int seg_end = e1 < lim ? e1 : lim;
                     const bool row_done = seg_end == e1;
                     if constexpr (X_LDS && NB == 1) {
@@ -489,10 +631,10 @@ __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1, int XF = 0>
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1, int XF = 0, bool ROWS = false>
 int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF>;
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF, ROWS>;
     const u32 n_waves = (u32)grid * (BLOCK / kWave);
     {
         // the sum the waves share evenly: stored entries plus row_cost per row (kept below 2^31)
@@ -527,6 +669,15 @@ int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
 // row): 5 to 9 % faster than cuts on entries alone; matrices of equal rows do not change.
 constexpr u32 kRowCost = 512;
 
+// Row ends in (what is left of) a tile from which on the tile is worked in one pass over all its rows.
+constexpr u32 kRowsPassMin = 3;
+// Mean stored entries per row below which the variant with that pass is launched.
+constexpr int kRowsPassBelow = 192;
+// ... and rows per wave from which on: the pass costs three round trips to LDS, which a wave with
+// a handful of rows in its only tile cannot hide (20000 x 300 at density 0.02, 32 rows per wave:
+// 15.0 -> 8.0 us; 5000 x 64 at 0.5, 8 rows: 10.0 -> 7.6 us; 1000 x 1000 at 0.05, 3 rows: 6.0 -> 6.4 us).
+constexpr long long kRowsPassRowsPerWave = 6;
+
 #ifdef MACKO_DEV_HOOKS
 // Launch-shape overrides for tuning runs (0 = built-in default); development builds only.
 struct Tuning {
@@ -534,8 +685,9 @@ struct Tuning {
     int grid;   // workgroups
     int split;  // 1: always the split kernel, -1: never
     int row_cost;  // what a row weighs in the cuts, in entries (-1: built-in)
+    int rows_pass_min;  // row ends in a tile from which on the tile is worked in one pass (-1: built-in, 0: never)
 };
-Tuning g_tuning = {0, 0, 0};
+Tuning g_tuning = {0, 0, 0, -1, -1};
 long long *g_trace = nullptr;
 #endif
 
@@ -609,6 +761,24 @@ int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
         return launch_stream<1024, 1, true, false, 2, NB>(a, (int)grid, lds_x, stream);
     }
     if (!fits) return launch_stream<1024, 2, false, AXPBY, VB>(a, (int)grid, 0, stream);
+    // Short rows (several ends per tile on average): the variant that works all the rows of a tile in
+    // one pass, if there is room for its 2 KB per wave behind x.
+    const size_t lds_rows = (lds_x + 15) & ~(size_t)15;
+    const size_t lds_all = lds_rows + (size_t)waves * kTile * 4;
+    bool rows_variant = a.padded < (long long)kRowsPassBelow * a.rows && (long long)a.rows >= kRowsPassRowsPerWave * grid * waves &&
+                        lds_all <= (size_t)info.max_lds_bytes;
+    a.rows_pass_min = kRowsPassMin;
+#ifdef MACKO_DEV_HOOKS
+    if (g_tuning.rows_pass_min >= 0) {
+        rows_variant = g_tuning.rows_pass_min > 0 && lds_all <= (size_t)info.max_lds_bytes;
+        a.rows_pass_min = (u32)g_tuning.rows_pass_min;
+    }
+#endif
+    if (rows_variant) {
+        a.rows_pass_lds = (u32)lds_rows;
+        if (depth == 2) return launch_stream<1024, 2, true, AXPBY, VB, 1, 0, true>(a, (int)grid, lds_all, stream);
+        return launch_stream<1024, 1, true, AXPBY, VB, 1, 0, true>(a, (int)grid, lds_all, stream);
+    }
     if (depth == 2) return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
     return launch_stream<1024, 1, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
 }
@@ -640,7 +810,10 @@ int check_spmv_args(const void *values, const void *deltas, const int32_t *row_p
 extern "C" void macko_spmv_set_trace(long long *device_buffer) { macko::g_trace = device_buffer; }
 extern "C" void macko_spmv_tune(int depth, int grid, int active, int split)
 {
-    macko::g_tuning = macko::Tuning{depth, grid, split, active > 0 ? active - 1 : -1};
+    // active: 0 = built-in values; else 1 + row_cost + 65536 * (1 + rows_pass_min)
+    const int row_cost = active > 0 ? ((active - 1) & 0xffff) : -1;
+    const int rows_pass_min = active > 0 ? ((active - 1) >> 16) - 1 : -1;
+    macko::g_tuning = macko::Tuning{depth, grid, split, row_cost, rows_pass_min};
 }
 #endif
 

@@ -52,6 +52,11 @@ struct SpmvArgs {
     // waves: the cuts balance entries + row_cost * rows (a row's end costs a reduction, a store and
     // masked passes, whatever its length).  entries_q / entries_rem then split that sum.
     u32 row_cost;
+    // Whole-row kernel, variant for short rows only.  What is left of a tile when at least
+    // rows_pass_min more rows end in it is worked in one pass over all those rows; that pass keeps
+    // 2 KB per wave in LDS, rows_pass_lds bytes into the dynamic LDS.
+    u32 rows_pass_min;
+    u32 rows_pass_lds;
 #ifdef MACKO_DEV_HOOKS
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif

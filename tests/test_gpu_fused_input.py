@@ -73,9 +73,14 @@ def test_multiply_silu_mul_axpby(shape, density):
     out = macko_spmv.multiply_silu_mul_axpby(c, gate, up, C)
     assert out.data_ptr() == C.data_ptr()
     helpers.assert_close_fp16(C.cpu().numpy(), product)
-    # same vector as the separate kernel builds, so the same sums in the same order
+    # same vector as the separate kernel builds, so the same sums in the same order; except for
+    # matrices of short rows, where the plain product adds a row's entries in another order (it works
+    # all the rows of a tile in one pass; the fused entry points have no such variant)
     unfused = macko_spmv.multiply(c, torch.ops.macko_spmv.decode_silu_mul(gate, up))
-    assert torch.equal(C, unfused)
+    if c[0].numel() >= 192 * rows:
+        assert torch.equal(C, unfused)
+    else:
+        assert torch.allclose(C.float(), unfused.float(), rtol=2e-3, atol=2e-4)
     # with the residual folded in
     C = torch.from_numpy(y0.copy()).cuda()
     macko_spmv.multiply_silu_mul_axpby(c, gate, up, C, alpha=0.5, beta=-2.0)
