@@ -118,10 +118,20 @@ spmv_stream_kernel(const SpmvArgs a)
         xpiece_issue<0>((u32)tid * 16, buf_x);
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
+    // Tile t of mine holds entries [tile_origin + 512 t, tile_origin + 512 (t + 1)).  Where a wave has
+    // few tiles (D == 1) they are counted from its own first entry, rounded down to a lane's 8
+    // entries: on the array's own grid nearly every wave would start in the middle of a tile and
+    // have one more tile to load and one more pass to make for the same entries (rows of 500
+    // entries, one to three per wave: 5 % per launch).  Long streams (D == 2) keep to the array's
+    // grid: there the loads that do not start on a cache line cost more than the extra tile (3 to
+    // 7 % per launch measured at density 0.5).
+    constexpr u32 kOriginAlign = D == 1 ? kChunk : kTile;
+    u32 tile_origin = 0;
     auto issue_slot = [&](auto slot, u32 tile, bool fetch, bool stream) {
         constexpr int J = decltype(slot)::value;
-        ring_issue<D, J, VB>(lane_values + (fetch ? tile * (u32)(kTile * VB) : kNoTileValues),
-                         lane4 + (fetch ? tile << (kTileShift - 1) : kNoTileDeltas), buf_values, buf_deltas, stream);
+        const u32 first = tile_origin + (tile << kTileShift);
+        ring_issue<D, J, VB>(lane_values + (fetch ? first * (u32)VB : kNoTileValues),
+                         lane4 + (fetch ? first >> 1 : kNoTileDeltas), buf_values, buf_deltas, stream);
     };
     // ---- 2. x: everything beyond the two register pieces per thread, and unaligned or odd-length
     //         x, goes to LDS through ordinary loads (rare: more than 16384 columns, or an x that is
@@ -263,10 +273,11 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 4. my tile range; the ring is filled with my first D tiles before x is even in LDS: they
     //         fly while the workgroup finishes the copy and meets at the barrier -------------------------
-    u32 first_tile = 0, last_tile = 0;
+    constexpr u32 first_tile = 0;
+    u32 last_tile = 0;
     if (__builtin_expect(have_work, 1)) {
-        first_tile = (u32)e0 >> kTileShift;
-        last_tile = ((u32)s_end + kTile - 1) >> kTileShift;  // exclusive
+        tile_origin = (u32)e0 & ~(kOriginAlign - 1);
+        last_tile = ((u32)s_end - tile_origin + kTile - 1) >> kTileShift;  // exclusive
         static_for<D>([&](auto slot) {
             constexpr int J = decltype(slot)::value;
             // my first and last tile may be shared with a neighbouring wave: no streaming hint there
@@ -567,7 +578,7 @@ spmv_stream_kernel(const SpmvArgs a)
             u32 dj;
             ring_take<D, J, kTileLoads - 2>(vj, dj);
             issue_slot(slot, tile + D, tile + D < last_tile, tile + D + 1 < last_tile);  // refill at once: the copy is out
-            const int tb = (int)(tile << kTileShift);
+            const int tb = (int)(tile_origin + (tile << kTileShift));
             const int tile_end = tb + kTile;
             if (e0 <= tb && e1 >= tile_end) {  // the common case for rows longer than a tile
                 full_tile_pass(vj, dj);
