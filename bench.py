@@ -160,7 +160,10 @@ def make_inputs(torch, suite):
 
 
 def clone_compressed(c):
-    return (c[0].clone(), c[1].clone(), c[2].clone(), c[3], c[4])
+    """A second copy of a compressed matrix, prepared like the first (compress attaches the product's
+    cuts to its result; a bare clone of the tensors would multiply without them)."""
+    import macko_spmv_amd
+    return macko_spmv_amd.attach_plan((c[0].clone(), c[1].clone(), c[2].clone(), c[3], c[4]))
 
 
 def time_graph(torch, fn, replays):

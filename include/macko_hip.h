@@ -66,6 +66,39 @@ MACKO_API int macko_spmv_f16_axpby(const void *values, const void *deltas, const
                          int64_t padded_entries, float alpha, float beta, void *stream);
 
 /*
+ * Prepared cuts ("plan") for macko_spmv_f16 / macko_spmv_f16_axpby.  No counterpart in the reference:
+ * its kernel owns one row per warp (src/macko_spmv/cuda/kernels.cuh:34-56) and has nothing to look
+ * up.  Here a launch deals whole rows to a fixed number of waves by stored entries, and every wave
+ * finds its first row in row_ptr when the kernel starts.  Where rows are about equally long that
+ * search takes one probe; where they are not (row lengths spread over orders of magnitude) it takes
+ * whole workgroups one or two more round trips to memory per launch.  A plan holds the result of
+ * that search for one matrix: build it once after compressing, pass it with every product.
+ *
+ *   macko_spmv_plan_entries  *entries = int32 elements a plan for this shape holds on the current
+ *                            device, 0 if products of this shape take none (no stored entries, fewer
+ *                            rows than waves, or a vector too long for LDS).
+ *   macko_spmv_plan_build    fills plan[0 .. plan_entries) from row_ptr; plan 16-byte aligned, device
+ *                            memory; plan_entries must be what macko_spmv_plan_entries returns.
+ *                            Asynchronous on `stream`.
+ *   macko_spmv_f16_planned, macko_spmv_f16_axpby_planned
+ *                            as macko_spmv_f16 / macko_spmv_f16_axpby.  A plan of another size than this
+ *                            launch needs (plan_entries 0, another device, another shape) is ignored
+ *                            and the rows are searched as usual; results are the same either way,
+ *                            bit for bit.  A plan built from another row_ptr is the caller's error,
+ *                            like a wrong row_ptr.
+ */
+MACKO_API int macko_spmv_plan_entries(int32_t rows, int32_t cols, int64_t padded_entries, int32_t *entries);
+MACKO_API int macko_spmv_plan_build(const int32_t *row_ptr, int32_t rows, int32_t cols,
+                          int64_t padded_entries, int32_t *plan, int32_t plan_entries, void *stream);
+MACKO_API int macko_spmv_f16_planned(const void *values, const void *deltas, const int32_t *row_ptr,
+                           const int32_t *plan, int32_t plan_entries, const void *x, void *y,
+                           int32_t rows, int32_t cols, int64_t padded_entries, void *stream);
+MACKO_API int macko_spmv_f16_axpby_planned(const void *values, const void *deltas, const int32_t *row_ptr,
+                                 const int32_t *plan, int32_t plan_entries, const void *x, void *y,
+                                 int32_t rows, int32_t cols, int64_t padded_entries, float alpha,
+                                 float beta, void *stream);
+
+/*
  * Compressor, step 1 of 2.  Reads the dense row-major fp16 matrix `dense` [rows, cols] and
  * writes row_ptr[0..rows] (int32, device).  Asynchronous.  The caller then reads
  * n = row_ptr[rows] back (one 4-byte copy + stream sync), sizes values/deltas to

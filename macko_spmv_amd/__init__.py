@@ -50,6 +50,16 @@ def _multiply_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V):
     return torch.empty((M_rows,), device=M_values.device, dtype=M_values.dtype)
 
 
+@torch.library.register_fake("macko_spmv::multiply_planned")
+def _multiply_planned_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, plan):
+    return torch.empty((M_rows,), device=M_values.device, dtype=M_values.dtype)
+
+
+@torch.library.register_fake("macko_spmv::multiply_axpby_planned")
+def _multiply_axpby_planned_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, V, C, alpha, beta, plan):
+    return None
+
+
 @torch.library.register_fake("macko_spmv::multiply_batched")
 def _multiply_batched_fake(M_values, M_deltas, M_row_indices, M_rows, M_cols, X):
     return torch.empty((X.shape[0], M_rows), device=M_values.device, dtype=M_values.dtype)
@@ -127,15 +137,38 @@ def _multiply_vmap(info, in_dims, M_values, M_deltas, M_row_indices, M_rows, M_c
 torch.library.register_vmap("macko_spmv::multiply", _multiply_vmap)
 
 
+# A compressed matrix on the GPU carries, as an attribute of its row_indices tensor, where every wave
+# of the product's launch starts (a "plan", torch.ops.macko_spmv.plan): `multiply` then has no rows to
+# search for.  The tuple keeps the upstream layout; a tuple without the attribute (tensors cloned, moved
+# or made elsewhere) multiplies the same, bit for bit, searching row_indices as it goes.  The tensors of
+# a compressed matrix are not to be modified in place.
+_PLAN_ATTRIBUTE = "_macko_spmv_plan"
+
+
+def attach_plan(compressed):
+    """Prepare the product's cuts for a compressed fp16 matrix on the GPU (once per matrix; `compress`
+    and `move_to_device` call this).  Returns `compressed`."""
+    values, _, row_indices, rows, cols = compressed[:5]
+    if row_indices.is_cuda and values.dtype == torch.float16:
+        plan = torch.ops.macko_spmv.plan.default(row_indices, rows, cols, values.numel())
+        setattr(row_indices, _PLAN_ATTRIBUTE, plan if plan.numel() else None)
+    return compressed
+
+
+def _plan_of(compressed):
+    plan = getattr(compressed[2], _PLAN_ATTRIBUTE, None)
+    return plan if plan is not None and plan.device == compressed[2].device else None
+
+
 def move_to_device(compressed, device):
     """Move the three tensors of a compressed matrix (src/macko_spmv/__init__.py:110-117)."""
-    return (
+    return attach_plan((
         compressed[0].to(device=device),
         compressed[1].to(device=device),
         compressed[2].to(device=device),
         compressed[3],
         compressed[4],
-    )
+    ))
 
 
 def compress(M):
@@ -148,7 +181,7 @@ def compress(M):
     """
     assert M.is_contiguous()
     if M.device.type in ("cuda", "cpu"):
-        return tuple(torch.ops.macko_spmv.compress.default(M))
+        return attach_plan(tuple(torch.ops.macko_spmv.compress.default(M)))
     raise NotImplementedError()
 
 
@@ -160,6 +193,9 @@ def multiply(compressed_M, V):
     assert compressed_M[2].is_cuda
     assert V.is_cuda
     assert V.is_contiguous()
+    plan = _plan_of(compressed_M)
+    if plan is not None:
+        return torch.ops.macko_spmv.multiply_planned.default(*compressed_M[:5], V, plan)
     return torch.ops.macko_spmv.multiply.default(
         compressed_M[0],
         compressed_M[1],
@@ -184,6 +220,10 @@ def multiply_axpby(compressed_M, V, C, alpha=1.0, beta=0.0):
     reuse_value_from_c instantiation (src/macko_spmv/cuda/kernels.cuh:113-118)."""
     assert compressed_M[0].is_cuda and V.is_cuda and C.is_cuda
     assert V.is_contiguous() and C.is_contiguous()
+    plan = _plan_of(compressed_M)
+    if plan is not None:
+        torch.ops.macko_spmv.multiply_axpby_planned.default(*compressed_M[:5], V, C, float(alpha), float(beta), plan)
+        return C
     torch.ops.macko_spmv.multiply_axpby.default(
         compressed_M[0], compressed_M[1], compressed_M[2], compressed_M[3], compressed_M[4], V, C,
         float(alpha), float(beta),

@@ -58,13 +58,18 @@ template <int D, int J, int N> __device__ __forceinline__ void ring_take(u32x4 &
 // short rows.  A variant of its own: compiled into the kernel, that pass costs the row loop of
 // every matrix 0.3 to 0.7 us per launch (measured on 4096 x 4096 and 11008 x 4096 at density 0.1),
 // used or not.
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB, int XF, bool ROWS>
+// PLAN = every wave reads where its rows start from a table the caller had built for this matrix
+// (a.plan, see macko_spmv_plan_build) instead of searching row_ptr for its cuts: the search costs
+// nothing where the rows are about equally long (its first probe hits), and one or two more round
+// trips to memory for whole workgroups where they are not.
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB, int NB, int XF, bool ROWS, bool PLAN>
 __global__ void __launch_bounds__(BLOCK) __attribute__((amdgpu_num_vgpr(kCompilerVgprs)))
 spmv_stream_kernel(const SpmvArgs a)
 {
     static_assert(NB == 1 || (NB <= 8 && X_LDS && !AXPBY && VB == 2), "batched variant: fp16, x in LDS, plain product");
     static_assert(XF == 0 || (NB == 1 && X_LDS && VB == 2), "fused staging: fp16, one vector, x in LDS");
     static_assert(!ROWS || (X_LDS && NB == 1 && XF == 0), "all rows of a tile in one pass: one vector, x in LDS");
+    static_assert(!PLAN || (X_LDS && NB == 1 && XF == 0), "prepared cuts: one vector, x in LDS");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     MACKO_RESERVE_FIXED_REGISTERS(MACKO_STREAM_FIXED_REGISTERS);
     constexpr int WAVES = BLOCK / kWave;
@@ -100,7 +105,16 @@ spmv_stream_kernel(const SpmvArgs a)
     // ---- 1. tracked loads, oldest first: row_ptr probes, x pieces ------------------------------------
     // probes: 64 consecutive row_ptr values around where my first / last row should be
     int target[2], base[2], guess[2];
-    {
+    int cut_row[2] = {0, 0}, cut_entry[2] = {0, 0};
+    if constexpr (PLAN) {
+        // {first row, its first entry} of wave gw and of wave gw + 1: one scalar load
+        const int4 cut = *reinterpret_cast<const int4 *>(a.plan + 2 * (size_t)gw);
+        cut_row[0] = cut.x;
+        cut_entry[0] = cut.y;
+        cut_row[1] = cut.z;
+        cut_entry[1] = cut.w;
+        target[0] = target[1] = guess[0] = guess[1] = base[1] = 0;
+    } else {
         target[0] = (int)even_split(gw, a.entries_q, a.entries_rem);  // < P < 2^31
         target[1] = (int)even_split(gw + 1, a.entries_q, a.entries_rem);
         guess[0] = (int)(gw * a.rows_q + __umulhi(gw, a.rows_frac));
@@ -117,6 +131,12 @@ spmv_stream_kernel(const SpmvArgs a)
     if (X_LDS && NB == 1 && XF == 0) {
         xpiece_issue<0>((u32)tid * 16, buf_x);
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
+    }
+    if constexpr (PLAN) {  // the window of row starts from my first row on, behind the x pieces
+        base[0] = cut_row[0];
+        int i0 = base[0] + lane;
+        i0 = i0 <= a.rows ? i0 : a.rows;
+        probe_issue<0>((u32)i0 * 4, buf_rows);
     }
     // Tile t of mine holds entries [tile_origin + 512 t, tile_origin + 512 (t + 1)).  Where a wave has
     // few tiles (D == 1) they are counted from its own first entry, rounded down to a lane's 8
@@ -141,9 +161,11 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 3. which rows are mine -----------------------------------------------------------------------
     constexpr int kXLoads = X_LDS && NB == 1 && XF == 0 ? kXRegs : 0;
-    int window[2];
-    window[0] = probe_take<0, kXLoads + 1>();
-    window[1] = probe_take<1, kXLoads>();
+    int window[2] = {0, 0};
+    if constexpr (!PLAN) {
+        window[0] = probe_take<0, kXLoads + 1>();
+        window[1] = probe_take<1, kXLoads>();
+    }
     // window of row_ptr values the row loop reads row starts from: lane i holds row_ptr[win_base + i]
     int win_base = base[0];
     int win = window[0];
@@ -178,7 +200,29 @@ spmv_stream_kernel(const SpmvArgs a)
     int r = 0;  // current row
     int e0 = 0, e1 = 0, s_end = 0;
     bool resolved = false;
-    {
+    constexpr u32 first_tile = 0;
+    u32 last_tile = 0;
+    auto fill_ring = [&]() __attribute__((always_inline)) {
+        tile_origin = (u32)e0 & ~(kOriginAlign - 1);
+        last_tile = ((u32)s_end - tile_origin + kTile - 1) >> kTileShift;  // exclusive
+        static_for<D>([&](auto slot) {
+            constexpr int J = decltype(slot)::value;
+            // my first and last tile may be shared with a neighbouring wave: no streaming hint there
+            issue_slot(slot, first_tile + J, first_tile + J < last_tile, J > 0 && first_tile + J + 1 < last_tile);
+        });
+    };
+    if constexpr (PLAN) {
+        r = uniform(cut_row[0]);
+        row_last = uniform(cut_row[1]);
+        e0 = uniform(cut_entry[0]);
+        s_end = uniform(cut_entry[1]);
+        have_work = r < row_last && e0 < s_end;
+        // nothing else stands between a wave and its tiles; the window of row starts is taken behind
+        // the barrier (it was requested last, and x must not wait for it)
+        if (__builtin_expect(have_work, 1)) fill_ring();
+        resolved = true;
+    }
+    if constexpr (!PLAN) {
         // Straight-line case: both cuts fall inside their probe windows and my first row is not
         // empty.  Cut k is the first row start at or after target k, or the one before it if that
         // is nearer (with rows of similar length every wave then gets the same number of rows).
@@ -273,16 +317,8 @@ spmv_stream_kernel(const SpmvArgs a)
 
     // ---- 4. my tile range; the ring is filled with my first D tiles before x is even in LDS: they
     //         fly while the workgroup finishes the copy and meets at the barrier -------------------------
-    constexpr u32 first_tile = 0;
-    u32 last_tile = 0;
-    if (__builtin_expect(have_work, 1)) {
-        tile_origin = (u32)e0 & ~(kOriginAlign - 1);
-        last_tile = ((u32)s_end - tile_origin + kTile - 1) >> kTileShift;  // exclusive
-        static_for<D>([&](auto slot) {
-            constexpr int J = decltype(slot)::value;
-            // my first and last tile may be shared with a neighbouring wave: no streaming hint there
-            issue_slot(slot, first_tile + J, first_tile + J < last_tile, J > 0 && first_tile + J + 1 < last_tile);
-        });
+    if constexpr (!PLAN) {
+        if (__builtin_expect(have_work, 1)) fill_ring();
     }
 
     // ---- 5. x pieces into LDS (older than the ring loads just issued, if any) ---------------------------
@@ -291,12 +327,14 @@ spmv_stream_kernel(const SpmvArgs a)
     } else if (X_LDS) {
         const u32 lds_x = (u32)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + kLdsFront;
         const u32 dst0 = lds_x + (u32)tid * 16, dst1 = dst0 + BLOCK * 16;
+        // (with PLAN the window's load stands between the x pieces and the ring)
+        constexpr int kBehindX = PLAN ? 1 : 0;
         if (__builtin_expect(have_work, 1)) {
-            if (tid < x_nvec) xpiece_to_lds<0, kTileLoads + 1>(dst0);
-            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, kTileLoads>(dst1);
+            if (tid < x_nvec) xpiece_to_lds<0, kTileLoads + kBehindX + 1>(dst0);
+            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, kTileLoads + kBehindX>(dst1);
         } else {
-            if (tid < x_nvec) xpiece_to_lds<0, 1>(dst0);
-            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, 0>(dst1);
+            if (tid < x_nvec) xpiece_to_lds<0, kBehindX + 1>(dst0);
+            if (tid + BLOCK < x_nvec) xpiece_to_lds<1, kBehindX>(dst1);
         }
         // the copies above are asm the compiler's wait tracking does not see
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -304,6 +342,26 @@ spmv_stream_kernel(const SpmvArgs a)
         __syncthreads();
     }
     MACKO_STAMP(4);
+    if constexpr (PLAN) {
+        if (__builtin_expect(have_work, 1)) {
+            win = probe_take<0, kTileLoads>();
+            e1 = row_start(r + 1);
+            while (e1 == e0) {  // first non-empty row; empty ones are written on the way
+                store_empty_row(r);
+                ++r;
+                slide_window(r);
+                e1 = row_start(r + 1);
+            }
+        } else {
+            win = probe_take<0, 0>();
+            // rows without a single entry: a zero each
+            for (int rr = r + lane; rr < row_last; rr += kWave) {
+                float out = 0.f;
+                if (AXPBY) out = a.beta * half_bits_to_float(a.y[rr]);
+                a.y[rr] = float_to_half_bits(out);
+            }
+        }
+    }
 
     if (__builtin_expect(!have_work, 0)) return;
 
@@ -642,22 +700,27 @@ __global__ void spmv_empty_kernel(uint16_t *y, int rows, float beta)
     if (r < rows) y[r] = AXPBY ? float_to_half_bits(beta * half_bits_to_float(y[r])) : (uint16_t)0;
 }
 
-template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1, int XF = 0, bool ROWS = false>
-int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
+// How the rows are dealt to n_waves owners: fills the fields of `a` the kernels (and the kernel that
+// prepares a plan) derive the cuts from.
+void set_cut_fields(SpmvArgs &a, u32 n_waves)
 {
-    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF, ROWS>;
-    const u32 n_waves = (u32)grid * (BLOCK / kWave);
-    {
-        // the sum the waves share evenly: stored entries plus row_cost per row (kept below 2^31)
-        const long long room = ((1ll << 31) - 1 - a.padded) / (a.rows > 0 ? a.rows : 1);
-        if ((long long)a.row_cost > room) a.row_cost = (u32)room;
-        const long long weight = a.padded + (long long)a.row_cost * a.rows;
-        a.entries_q = (u32)(weight / n_waves);
-        a.entries_rem = (u32)(weight % n_waves);
-    }
+    // the sum the waves share evenly: stored entries plus row_cost per row (kept below 2^31)
+    const long long room = ((1ll << 31) - 1 - a.padded) / (a.rows > 0 ? a.rows : 1);
+    if ((long long)a.row_cost > room) a.row_cost = (u32)room;
+    const long long weight = a.padded + (long long)a.row_cost * a.rows;
+    a.entries_q = (u32)(weight / n_waves);
+    a.entries_rem = (u32)(weight % n_waves);
     a.rows_q = (u32)a.rows / n_waves;
     a.rows_frac = (u32)(((unsigned long long)((u32)a.rows % n_waves) << 32) / n_waves);
     a.row_even = (u32)a.rows <= n_waves ? 1u : 0u;
+}
+
+template <int BLOCK, int D, bool X_LDS, bool AXPBY, int VB = 2, int NB = 1, int XF = 0, bool ROWS = false,
+          bool PLAN = false>
+int launch_stream(SpmvArgs a, int grid, size_t lds_bytes, hipStream_t stream)
+{
+    auto kernel = spmv_stream_kernel<BLOCK, D, X_LDS, AXPBY, VB, NB, XF, ROWS, PLAN>;
+    set_cut_fields(a, (u32)grid * (BLOCK / kWave));
     if (lds_bytes > 64 * 1024) {
         // one-time opt-in to more than 64 KiB of dynamic LDS, per device and kernel
         static std::atomic<bool> done[64];
@@ -702,6 +765,39 @@ Tuning g_tuning = {0, 0, 0, -1, -1};
 long long *g_trace = nullptr;
 #endif
 
+// The launch a matrix gets: workgroups of the whole-row kernel, or the split kernel.
+struct LaunchShape {
+    long long n_tiles;
+    long long grid;  // workgroups of 1024 threads of the whole-row kernel
+    bool split;      // rows are split between the waves of a workgroup instead (macko_spmv_split.hip)
+};
+
+LaunchShape launch_shape(int rows, long long padded, const DeviceInfo &info)
+{
+    constexpr int waves = 1024 / kWave;
+    LaunchShape s;
+    // about one wave per tile at most, so tiny matrices get a small grid; but when rows are about
+    // a tile long, prefer one wave per row over a slightly smaller wave count that would leave
+    // some waves with two rows
+    s.n_tiles = (padded + kTile - 1) / kTile;
+    long long waves_wanted = s.n_tiles;
+    if (rows > waves_wanted) waves_wanted = rows < 2 * s.n_tiles ? rows : 2 * s.n_tiles;
+    s.grid = (waves_wanted + waves - 1) / waves;
+    if (s.grid > (long long)info.compute_units) s.grid = (long long)info.compute_units;
+    if (s.grid < 1) s.grid = 1;
+    // Whole rows per wave need about as many rows as waves; with clearly fewer, the workgroups own
+    // the rows and their waves split them (macko_spmv_split.hip): one workgroup per compute unit,
+    // at least a tile per wave and a row per workgroup.
+    // Only where rows are long (four tiles and more on average): for short rows a wave per row is
+    // the cheaper way even if most waves stay idle.
+    s.split = 4 * (long long)rows < 3 * s.grid * waves && s.n_tiles >= 4 * (long long)rows;
+#ifdef MACKO_DEV_HOOKS
+    if (g_tuning.split) s.split = g_tuning.split > 0;
+    if (g_tuning.grid && !s.split) s.grid = g_tuning.grid;
+#endif
+    return s;
+}
+
 template <bool AXPBY, int VB = 2, int NB = 1, int XF = 0>
 int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
 {
@@ -717,23 +813,11 @@ int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
     if (rc != 0) return rc;
 
     constexpr int waves = 1024 / kWave;
-    // about one wave per tile at most, so tiny matrices get a small grid; but when rows are about
-    // a tile long, prefer one wave per row over a slightly smaller wave count that would leave
-    // some waves with two rows
-    const long long n_tiles = (a.padded + kTile - 1) / kTile;
-    long long waves_wanted = n_tiles;
-    if (a.rows > waves_wanted) waves_wanted = a.rows < 2 * n_tiles ? a.rows : 2 * n_tiles;
-    long long grid = (waves_wanted + waves - 1) / waves;
-    if (grid > (long long)info.compute_units) grid = (long long)info.compute_units;
-    if (grid < 1) grid = 1;
-    // Whole rows per wave need about as many rows as waves; with clearly fewer, the workgroups own
-    // the rows and their waves split them (macko_spmv_split.hip): one workgroup per compute unit,
-    // at least a tile per wave and a row per workgroup.
-    // Only where rows are long (four tiles and more on average): for short rows a wave per row is
-    // the cheaper way even if most waves stay idle.
-    bool split = 4 * (long long)a.rows < 3 * grid * waves && n_tiles >= 4 * (long long)a.rows;
+    const LaunchShape shape = launch_shape(a.rows, a.padded, info);
+    const long long n_tiles = shape.n_tiles;
+    long long grid = shape.grid;
+    const bool split = shape.split;
 #ifdef MACKO_DEV_HOOKS
-    if (g_tuning.split) split = g_tuning.split > 0;
     a.trace = g_trace;
 #endif
     const size_t lds_x = (size_t)NB * ((size_t)kLdsFront + 2 * (size_t)a.cols + kLdsBack) + (XF == 1 ? 64 : 0);
@@ -758,7 +842,6 @@ int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
 #ifdef MACKO_DEV_HOOKS
     if (g_tuning.row_cost >= 0) a.row_cost = (u32)g_tuning.row_cost;
     if (g_tuning.depth) depth = g_tuning.depth;
-    if (g_tuning.grid) grid = g_tuning.grid;
 #endif
     const bool fits = lds_x <= (size_t)info.max_lds_bytes;
     if (XF != 0) {  // fused staging: x must fit in LDS (checked by the caller too)
@@ -785,13 +868,77 @@ int spmv_dispatch(const SpmvArgs &args, hipStream_t stream)
         a.rows_pass_min = (u32)g_tuning.rows_pass_min;
     }
 #endif
+    // A plan is used if it was built for exactly this launch (same number of waves); any other is ignored.
+    const bool planned = VB == 2 && a.plan != nullptr && (long long)a.plan_entries == 2 * (grid * waves + 1);
     if (rows_variant) {
         a.rows_pass_lds = (u32)lds_rows;
+        if constexpr (VB == 2) {
+            if (planned) {
+                if (depth == 2) return launch_stream<1024, 2, true, AXPBY, 2, 1, 0, true, true>(a, (int)grid, lds_all, stream);
+                return launch_stream<1024, 1, true, AXPBY, 2, 1, 0, true, true>(a, (int)grid, lds_all, stream);
+            }
+        }
         if (depth == 2) return launch_stream<1024, 2, true, AXPBY, VB, 1, 0, true>(a, (int)grid, lds_all, stream);
         return launch_stream<1024, 1, true, AXPBY, VB, 1, 0, true>(a, (int)grid, lds_all, stream);
     }
+    if constexpr (VB == 2) {
+        if (planned) {
+            if (depth == 2) return launch_stream<1024, 2, true, AXPBY, 2, 1, 0, false, true>(a, (int)grid, lds_x, stream);
+            return launch_stream<1024, 1, true, AXPBY, 2, 1, 0, false, true>(a, (int)grid, lds_x, stream);
+        }
+    }
     if (depth == 2) return launch_stream<1024, 2, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
     return launch_stream<1024, 1, true, AXPBY, VB>(a, (int)grid, lds_x, stream);
+}
+
+// One thread per cut: cut k is where wave k of the launch starts (cut n_waves: the end), by the
+// rule the kernel itself applies when it has no plan: the first row r with
+// row_ptr[r] + row_cost * r >= target k, or the row before if that is nearer; even shares of the
+// rows when there are no more rows than waves.  plan[2k] = row, plan[2k + 1] = row_ptr[row].
+__global__ void plan_kernel(const SpmvArgs a, u32 n_waves, int *__restrict__ plan)
+{
+    const u32 k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k > n_waves) return;
+    int cut;
+    if (k == 0) {
+        cut = 0;
+    } else if (k == n_waves) {
+        cut = a.rows;
+    } else if (a.row_even) {
+        cut = (int)(k * a.rows_q + __umulhi(k, a.rows_frac));
+    } else {
+        const long long target = (long long)even_split(k, a.entries_q, a.entries_rem);
+        const long long row_cost = (long long)a.row_cost;
+        int lo = 0, hi = a.rows;  // cost(rows) = the whole sum >= any target
+        while (lo < hi) {
+            const int mid = lo + ((hi - lo) >> 1);
+            if ((long long)a.row_ptr[mid] + row_cost * mid >= target) hi = mid; else lo = mid + 1;
+        }
+        cut = lo;
+        if (cut > 0) {
+            const long long after = (long long)a.row_ptr[cut] + row_cost * cut;
+            const long long before = (long long)a.row_ptr[cut - 1] + row_cost * (cut - 1);
+            if (target - before < after - target) cut -= 1;
+        }
+    }
+    plan[2 * k] = cut;
+    plan[2 * k + 1] = a.row_ptr[cut];
+}
+
+// Waves of the launch a plan describes, 0 if this shape takes none (no stored entries, rows split
+// between waves, or x too long for LDS).
+int plan_waves(int rows, int cols, long long padded, long long *n_waves)
+{
+    *n_waves = 0;
+    if (rows == 0 || padded == 0) return 0;
+    DeviceInfo info;
+    const int rc = device_info(&info);
+    if (rc != 0) return rc;
+    const LaunchShape shape = launch_shape(rows, padded, info);
+    const size_t lds_x = (size_t)kLdsFront + 2 * (size_t)cols + kLdsBack;
+    if (shape.split || lds_x > (size_t)info.max_lds_bytes) return 0;
+    *n_waves = shape.grid * (1024 / kWave);
+    return 0;
 }
 
 // LDS the split kernel keeps behind x at most (16 waves, up to 8 vectors and a flag each)
@@ -852,6 +999,98 @@ extern "C" int macko_spmv_f16_axpby(const void *values, const void *deltas, cons
                rows,                cols,                padded_entries, alpha,         beta,
                0,                   0,                   0,              0,             0,
                0,                   0};
+    return spmv_dispatch<true>(a, as_stream(stream));
+}
+
+// ---- prepared cuts (no counterpart upstream) ------------------------------------------------------
+extern "C" int macko_spmv_plan_entries(int32_t rows, int32_t cols, int64_t padded_entries, int32_t *entries)
+{
+    using namespace macko;
+    if (entries == nullptr || rows < 0 || cols < 0 || padded_entries < 0) return MACKO_E_INVALID_ARGUMENT;
+    long long n_waves = 0;
+    const int rc = plan_waves(rows, cols, padded_entries, &n_waves);
+    *entries = n_waves > 0 ? (int32_t)(2 * (n_waves + 1)) : 0;
+    return rc;
+}
+
+extern "C" int macko_spmv_plan_build(const int32_t *row_ptr, int32_t rows, int32_t cols, int64_t padded_entries,
+                                     int32_t *plan, int32_t plan_entries, void *stream)
+{
+    using namespace macko;
+    if (rows < 0 || cols < 0 || padded_entries < 0 || padded_entries % kChunk != 0 ||
+        padded_entries >= (1ll << 31) - 8192)
+        return MACKO_E_INVALID_ARGUMENT;
+    long long n_waves = 0;
+    const int rc = plan_waves(rows, cols, padded_entries, &n_waves);
+    if (rc != 0) return rc;
+    if ((long long)plan_entries != (n_waves > 0 ? 2 * (n_waves + 1) : 0)) return MACKO_E_INVALID_ARGUMENT;
+    if (n_waves == 0) return 0;
+    if (row_ptr == nullptr || plan == nullptr || (reinterpret_cast<uintptr_t>(row_ptr) & 3) ||
+        (reinterpret_cast<uintptr_t>(plan) & 15))
+        return MACKO_E_INVALID_ARGUMENT;
+    SpmvArgs a{};
+    a.row_ptr = row_ptr;
+    a.rows = rows;
+    a.cols = cols;
+    a.padded = padded_entries;
+    a.row_cost = kRowCost;
+#ifdef MACKO_DEV_HOOKS
+    if (g_tuning.row_cost >= 0) a.row_cost = (u32)g_tuning.row_cost;
+#endif
+    set_cut_fields(a, (u32)n_waves);
+    const int threads = 256;
+    hipLaunchKernelGGL(plan_kernel, dim3((unsigned)((n_waves + 1 + threads - 1) / threads)), dim3(threads), 0,
+                       as_stream(stream), a, (u32)n_waves, plan);
+    return (int)hipGetLastError();
+}
+
+extern "C" int macko_spmv_f16_planned(const void *values, const void *deltas, const int32_t *row_ptr,
+                                      const int32_t *plan, int32_t plan_entries, const void *x, void *y,
+                                      int32_t rows, int32_t cols, int64_t padded_entries, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
+    if (rc != 0) return rc;
+    if (plan_entries < 0 || (plan_entries > 0 && (plan == nullptr || (reinterpret_cast<uintptr_t>(plan) & 15))))
+        return MACKO_E_INVALID_ARGUMENT;
+    SpmvArgs a{};
+    a.values = (const u32 *)values;
+    a.deltas = (const u32 *)deltas;
+    a.row_ptr = row_ptr;
+    a.x = (const uint16_t *)x;
+    a.y = (uint16_t *)y;
+    a.rows = rows;
+    a.cols = cols;
+    a.padded = padded_entries;
+    a.alpha = 1.0f;
+    a.plan = plan_entries > 0 ? plan : nullptr;
+    a.plan_entries = plan_entries;
+    return spmv_dispatch<false>(a, as_stream(stream));
+}
+
+extern "C" int macko_spmv_f16_axpby_planned(const void *values, const void *deltas, const int32_t *row_ptr,
+                                            const int32_t *plan, int32_t plan_entries, const void *x, void *y,
+                                            int32_t rows, int32_t cols, int64_t padded_entries, float alpha,
+                                            float beta, void *stream)
+{
+    using namespace macko;
+    int rc = check_spmv_args(values, deltas, row_ptr, x, y, rows, cols, padded_entries);
+    if (rc != 0) return rc;
+    if (plan_entries < 0 || (plan_entries > 0 && (plan == nullptr || (reinterpret_cast<uintptr_t>(plan) & 15))))
+        return MACKO_E_INVALID_ARGUMENT;
+    SpmvArgs a{};
+    a.values = (const u32 *)values;
+    a.deltas = (const u32 *)deltas;
+    a.row_ptr = row_ptr;
+    a.x = (const uint16_t *)x;
+    a.y = (uint16_t *)y;
+    a.rows = rows;
+    a.cols = cols;
+    a.padded = padded_entries;
+    a.alpha = alpha;
+    a.beta = beta;
+    a.plan = plan_entries > 0 ? plan : nullptr;
+    a.plan_entries = plan_entries;
     return spmv_dispatch<true>(a, as_stream(stream));
 }
 

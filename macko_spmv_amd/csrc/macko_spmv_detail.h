@@ -57,6 +57,10 @@ struct SpmvArgs {
     // 2 KB per wave in LDS, rows_pass_lds bytes into the dynamic LDS.
     u32 rows_pass_min;
     u32 rows_pass_lds;
+    // Whole-row kernel with prepared cuts only: {first row, its first entry} per wave of the launch
+    // and one more pair for the end (rows, stored entries), as macko_spmv_plan_build writes them.
+    const int *plan;
+    int plan_entries;  // host side only: int32 elements behind `plan`, 2 * (waves of the launch + 1)
 #ifdef MACKO_DEV_HOOKS
     long long *trace;  // 8 timestamps per wave (development builds only)
 #endif

@@ -67,6 +67,71 @@ at::Tensor multiply_hip(const at::Tensor &M_values, const at::Tensor &M_deltas, 
     return C;
 }
 
+// Where every wave of the product's launch starts (macko_spmv_plan_build): int32 [entries], empty if
+// products of this shape take none.  Built once per matrix, after compressing.
+at::Tensor plan_hip(const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, int64_t padded_entries)
+{
+    TORCH_CHECK(M_row_indices.dtype() == at::kInt && M_row_indices.is_cuda() && M_row_indices.is_contiguous(),
+                "M_row_indices must be a contiguous torch.int32 GPU tensor");
+    TORCH_CHECK(M_rows >= 0 && M_cols >= 0 && M_rows < (1ll << 31) && M_cols < (1ll << 31), "bad dimensions");
+    TORCH_CHECK(M_row_indices.numel() >= M_rows + 1, "M_row_indices must hold M_rows + 1 elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_row_indices.device());
+    int32_t entries = 0;
+    check_rc(macko_spmv_plan_entries((int32_t)M_rows, (int32_t)M_cols, padded_entries, &entries), "plan");
+    at::Tensor plan = at::empty({entries}, M_row_indices.options());
+    if (entries == 0) return plan;
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    check_rc(macko_spmv_plan_build(M_row_indices.data_ptr<int>(), (int32_t)M_rows, (int32_t)M_cols, padded_entries,
+                                   plan.data_ptr<int>(), entries, (void *)stream),
+             "plan");
+    return plan;
+}
+
+void check_plan(const at::Tensor &plan, const at::Tensor &M_values)
+{
+    TORCH_CHECK(plan.dtype() == at::kInt && plan.is_contiguous(), "plan must be a contiguous torch.int32 tensor");
+    TORCH_CHECK(plan.numel() == 0 || (plan.is_cuda() && plan.device() == M_values.device()),
+                "plan must live on the matrix's GPU");
+}
+
+at::Tensor multiply_planned_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                                const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &V,
+                                const at::Tensor &plan)
+{
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(V, "V");
+    check_plan(plan, M_values);
+    TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    at::Tensor C = at::empty({M_rows}, M_values.options());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const int rc = macko_spmv_f16_planned(M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+                                          plan.numel() ? plan.data_ptr<int>() : nullptr, (int32_t)plan.numel(),
+                                          V.data_ptr(), C.data_ptr(), (int32_t)M_rows, (int32_t)M_cols,
+                                          M_values.numel(), (void *)stream);
+    check_rc(rc, "multiply_planned");
+    return C;
+}
+
+void multiply_axpby_planned_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
+                                const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &V,
+                                at::Tensor C, double alpha, double beta, const at::Tensor &plan)
+{
+    check_macko_operands(M_values, M_deltas, M_row_indices, M_rows, M_cols);
+    check_half_gpu(V, "V");
+    check_half_gpu(C, "C");
+    check_plan(plan, M_values);
+    TORCH_CHECK(C.numel() >= M_rows, "C must hold M_rows elements");
+    TORCH_CHECK(V.numel() >= M_cols || M_values.numel() == 0, "V must hold at least M_cols elements");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(M_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const int rc = macko_spmv_f16_axpby_planned(
+        M_values.data_ptr(), M_deltas.data_ptr(), M_row_indices.data_ptr<int>(),
+        plan.numel() ? plan.data_ptr<int>() : nullptr, (int32_t)plan.numel(), V.data_ptr(), C.data_ptr(),
+        (int32_t)M_rows, (int32_t)M_cols, M_values.numel(), (float)alpha, (float)beta, (void *)stream);
+    check_rc(rc, "multiply_axpby_planned");
+}
+
 // Y[b] = M @ X[b] for X of shape [batch, M_cols] -> [batch, M_rows].
 at::Tensor multiply_batched_hip(const at::Tensor &M_values, const at::Tensor &M_deltas,
                                 const at::Tensor &M_row_indices, int64_t M_rows, int64_t M_cols, const at::Tensor &X)
@@ -411,6 +476,11 @@ TORCH_LIBRARY(macko_spmv, m)
           "Tensor X) -> Tensor");
     m.def("multiply_axpby(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
           "Tensor V, Tensor(a!) C, float alpha, float beta) -> ()");
+    m.def("plan(Tensor M_row_indices, int M_rows, int M_cols, int padded_entries) -> Tensor");
+    m.def("multiply_planned(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V, Tensor plan) -> Tensor");
+    m.def("multiply_axpby_planned(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
+          "Tensor V, Tensor(a!) C, float alpha, float beta, Tensor plan) -> ()");
     m.def("compress(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
     m.def("compress_int8(Tensor M) -> (Tensor, Tensor, Tensor, int, int)");
     m.def("multiply_int8(Tensor M_values, Tensor M_deltas, Tensor M_row_indices, int M_rows, int M_cols, "
@@ -436,6 +506,9 @@ TORCH_LIBRARY_IMPL(macko_spmv, CUDA, m)
     m.impl("multiply", &multiply_hip);
     m.impl("multiply_batched", &multiply_batched_hip);
     m.impl("multiply_axpby", &multiply_axpby_hip);
+    m.impl("plan", &plan_hip);
+    m.impl("multiply_planned", &multiply_planned_hip);
+    m.impl("multiply_axpby_planned", &multiply_axpby_planned_hip);
     m.impl("compress", &compress_hip);
     m.impl("compress_int8", &compress_int8_hip);
     m.impl("multiply_int8", &multiply_int8_hip);
