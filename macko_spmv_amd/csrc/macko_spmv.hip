@@ -138,14 +138,15 @@ spmv_stream_kernel(const SpmvArgs a)
         i0 = i0 <= a.rows ? i0 : a.rows;
         probe_issue<0>((u32)i0 * 4, buf_rows);
     }
-    // Tile t of mine holds entries [tile_origin + 512 t, tile_origin + 512 (t + 1)).  Where a wave has
-    // few tiles (D == 1) they are counted from its own first entry, rounded down to a lane's 8
-    // entries: on the array's own grid nearly every wave would start in the middle of a tile and
-    // have one more tile to load and one more pass to make for the same entries (rows of 500
-    // entries, one to three per wave: 5 % per launch).  Long streams (D == 2) keep to the array's
-    // grid: there the loads that do not start on a cache line cost more than the extra tile (3 to
-    // 7 % per launch measured at density 0.5).
-    constexpr u32 kOriginAlign = D == 1 ? kChunk : kTile;
+    // Tile t of mine holds entries [tile_origin + 512 t, tile_origin + 512 (t + 1)).  My tiles are
+    // counted from my own first entry, not on a grid of the whole array's: there nearly every wave
+    // would start in the middle of a tile and have one more tile to load and one more pass to make
+    // for the same entries.  Where a wave has few tiles (D == 1) the origin is rounded down to a
+    // lane's 8 entries only (rows of 500 entries, one to three per wave: 5 % per launch).  Long
+    // streams (D == 2) round it down to 256 entries, so that every load still starts on a cache
+    // line (128 bytes of nibbles): loads that do not cost them more than the tile they save (3 to
+    // 7 % per launch at density 0.5 with an origin rounded to 8; 1 to 3 % gained with 256).
+    constexpr u32 kOriginAlign = D == 1 ? kChunk : 256;
     u32 tile_origin = 0;
     auto issue_slot = [&](auto slot, u32 tile, bool fetch, bool stream) {
         constexpr int J = decltype(slot)::value;
