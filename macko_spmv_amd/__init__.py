@@ -137,6 +137,16 @@ def _multiply_vmap(info, in_dims, M_values, M_deltas, M_row_indices, M_rows, M_c
 torch.library.register_vmap("macko_spmv::multiply", _multiply_vmap)
 
 
+def _multiply_planned_vmap(info, in_dims, M_values, M_deltas, M_row_indices, M_rows, M_cols, V, plan):
+    # the batched product has no use for the single-vector launch's cuts
+    if in_dims[6] is not None:
+        raise NotImplementedError("macko_spmv::multiply_planned: vmap is supported over V only")
+    return _multiply_vmap(info, in_dims[:6], M_values, M_deltas, M_row_indices, M_rows, M_cols, V)
+
+
+torch.library.register_vmap("macko_spmv::multiply_planned", _multiply_planned_vmap)
+
+
 # A compressed matrix on the GPU carries, as an attribute of its row_indices tensor, where every wave
 # of the product's launch starts (a "plan", torch.ops.macko_spmv.plan): `multiply` then has no rows to
 # search for.  The tuple keeps the upstream layout; a tuple without the attribute (tensors cloned, moved

@@ -427,7 +427,10 @@ def test_vmap_over_the_vector_like_the_upstream_llm_layer():
     c = macko_spmv.compress(M)
     lifted = torch.vmap(lambda x: macko_spmv.multiply(c, x), in_dims=-2, out_dims=-2)
     x = torch.randn(1, 6, 700, device="cuda", dtype=torch.float16)
-    out = lifted(x)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")   # no fall-back to a loop over the batch: one batched product
+        out = lifted(x)
     assert out.shape == (6, 300)
     assert torch.allclose(out.float(), x[0].float() @ M.float().t(), rtol=1e-2, atol=2e-2)
 
