@@ -133,7 +133,7 @@ spmv_stream_kernel(const SpmvArgs a)
         xpiece_issue<1>((u32)(tid + BLOCK) * 16, buf_x);
     }
     if constexpr (PLAN) {  // the window of row starts from my first row on, behind the x pieces
-        base[0] = cut_row[0];
+        base[0] = (int)((u32)cut_row[0] < (u32)a.rows ? (u32)cut_row[0] : (u32)a.rows);
         int i0 = base[0] + lane;
         i0 = i0 <= a.rows ? i0 : a.rows;
         probe_issue<0>((u32)i0 * 4, buf_rows);
@@ -213,10 +213,16 @@ spmv_stream_kernel(const SpmvArgs a)
         });
     };
     if constexpr (PLAN) {
-        r = uniform(cut_row[0]);
-        row_last = uniform(cut_row[1]);
-        e0 = uniform(cut_entry[0]);
-        s_end = uniform(cut_entry[1]);
+        // (clamped, so that a plan that does not belong to this matrix can make the result wrong
+        // but no access leave the arrays and no loop run longer than the matrix is)
+        // (unsigned minimum: a negative value counts as too large)
+        auto at_most = [](int v, int most) { return (int)((u32)v < (u32)most ? (u32)v : (u32)most); };
+        r = at_most(uniform(cut_row[0]), a.rows);
+        row_last = at_most(uniform(cut_row[1]), a.rows);
+        row_last = row_last < r ? r : row_last;
+        e0 = at_most(uniform(cut_entry[0]), (int)a.padded);
+        s_end = at_most(uniform(cut_entry[1]), (int)a.padded);
+        s_end = s_end < e0 ? e0 : s_end;
         have_work = r < row_last && e0 < s_end;
         // nothing else stands between a wave and its tiles; the window of row starts is taken behind
         // the barrier (it was requested last, and x must not wait for it)
@@ -347,7 +353,7 @@ spmv_stream_kernel(const SpmvArgs a)
         if (__builtin_expect(have_work, 1)) {
             win = probe_take<0, kTileLoads>();
             e1 = row_start(r + 1);
-            while (e1 == e0) {  // first non-empty row; empty ones are written on the way
+            while (e1 == e0 && r + 1 < row_last) {  // first non-empty row; empty ones are written on the way
                 store_empty_row(r);
                 ++r;
                 slide_window(r);
@@ -492,7 +498,15 @@ spmv_stream_kernel(const SpmvArgs a)
         row_addr = row_origin;
         do {  // next non-empty owned row; empty ones get their zero on the way
             ++r;
-            if (r >= row_last) break;  // then the row just finished ended at s_end and all loops end
+            if (r >= row_last) {
+                // The row just finished ended at s_end and all loops end.  With a row_ptr that runs
+                // backwards, or cuts that are not this matrix's, entries may seem to be left: no
+                // row claims them (every later step then sees a row that starts at infinity, which
+                // writes nothing and moves on), so the walk ends whatever the arrays hold.
+                e0 = e1 = 0x7fffffff;
+                last_tile = 0;
+                break;
+            }
             slide_window(r);
             e0 = row_start(r);
             e1 = row_start(r + 1);
@@ -613,7 +627,11 @@ spmv_stream_kernel(const SpmvArgs a)
         r = open_row - 1;
         do {
             ++r;
-            if (r >= row_last) break;
+            if (r >= row_last) {  // as in finish_row
+                e0 = e1 = 0x7fffffff;
+                last_tile = 0;
+                break;
+            }
             slide_window(r);
             e0 = row_start(r);
             e1 = row_start(r + 1);
@@ -653,6 +671,10 @@ spmv_stream_kernel(const SpmvArgs a)
                             const int known = row_last < win_base + 63 ? row_last : win_base + 63;
                             const int known_start = row_start(known);
                             const int stop = known_start < lim ? known_start : lim;
+                            if (__builtin_expect(stop <= pos, 0)) {  // see below: only a broken row_ptr does this
+                                last_tile = 0;
+                                break;
+                            }
                             rows_pass(vj, dj, tb, pos, stop);
                             pos = stop;
                             continue;

@@ -163,3 +163,37 @@ def test_move_to_device_attaches_a_plan_and_graphs_replay_with_it():
             stream.synchronize()
             assert torch.equal(out, eager)
     torch.cuda.current_stream().wait_stream(stream)
+
+
+def test_a_plan_that_is_not_this_matrix_s_stays_inside_the_arrays():
+    # the kernel clamps what it reads from a plan and ends its walk when the rows stop making sense:
+    # the product is then wrong, but the call returns, y beyond `rows` is untouched and the next
+    # product is right
+    rng = np.random.default_rng(23)
+    rows, cols = 6000, 1024
+    dense = _skewed(rng, rows, cols)
+    x = rng.standard_normal(cols).astype(np.float16)
+    c = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    xg = torch.from_numpy(x).cuda()
+    lib = _lib()
+    P = c[0].numel()
+    good = getattr(c[2], "_macko_spmv_plan")
+    n = good.numel()
+    cuts = good.view(-1, 2)
+    wrong_plans = {
+        "reversed": cuts.flip(0).contiguous().view(-1),
+        "zeros": torch.zeros_like(good),
+        "huge": torch.full_like(good, 1 << 30),
+        "negative": torch.full_like(good, -5),
+        "rows and entries swapped": cuts.flip(1).contiguous().view(-1),
+        "entries of another place": torch.stack([cuts[:, 0], cuts[:, 1].roll(7)], dim=1).contiguous().view(-1),
+    }
+    for label, plan in wrong_plans.items():
+        print("wrong plan:", label, flush=True)
+        y = torch.full((rows + 64,), 3.0, dtype=torch.float16, device="cuda")
+        assert lib.macko_spmv_f16_planned(c[0].data_ptr(), c[1].data_ptr(), c[2].data_ptr(), plan.data_ptr(), n,
+                                          xg.data_ptr(), y.data_ptr(), rows, cols, P, None) == 0
+        torch.cuda.synchronize()
+        assert bool((y[rows:] == 3.0).all())
+    y = macko_spmv.multiply(c, xg)
+    helpers.assert_close_fp16(y.cpu().numpy(), helpers.dense_reference(dense, x))
