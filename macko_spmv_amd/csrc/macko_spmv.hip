@@ -205,7 +205,10 @@ spmv_stream_kernel(const SpmvArgs a)
     u32 last_tile = 0;
     auto fill_ring = [&]() __attribute__((always_inline)) {
         tile_origin = (u32)e0 & ~(kOriginAlign - 1);
-        last_tile = ((u32)s_end - tile_origin + kTile - 1) >> kTileShift;  // exclusive
+        // (exclusive; none if my rows end in front of where they start, and none beyond the arrays:
+        // a row_ptr that runs backwards or points outside cannot make the walk longer than the matrix)
+        const int end = s_end < (int)a.padded ? s_end : (int)a.padded;
+        last_tile = end > e0 ? ((u32)end - tile_origin + kTile - 1) >> kTileShift : 0u;
         static_for<D>([&](auto slot) {
             constexpr int J = decltype(slot)::value;
             // my first and last tile may be shared with a neighbouring wave: no streaming hint there

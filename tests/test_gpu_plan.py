@@ -197,3 +197,38 @@ def test_a_plan_that_is_not_this_matrix_s_stays_inside_the_arrays():
         assert bool((y[rows:] == 3.0).all())
     y = macko_spmv.multiply(c, xg)
     helpers.assert_close_fp16(y.cpu().numpy(), helpers.dense_reference(dense, x))
+
+
+def test_a_row_ptr_that_makes_no_sense_stays_inside_the_arrays():
+    # same promise for the kernel's own search (no plan): wrong row_ptr, wrong product, but the call
+    # returns and nothing outside y[0 .. rows) is written.  (Shapes whose rows are split between the
+    # waves of a workgroup are not part of this test.)
+    rng = np.random.default_rng(29)
+    rows, cols = 6000, 1024
+    dense = helpers.random_sparse(rng, rows, cols, 0.3)
+    x = rng.standard_normal(cols).astype(np.float16)
+    c = macko_spmv.compress(torch.from_numpy(dense).cuda())
+    xg = torch.from_numpy(x).cuda()
+    lib = _lib()
+    P = c[0].numel()
+    good = c[2]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    wrong = {
+        "reversed": good.flip(0).contiguous(),
+        "all zero": torch.zeros_like(good),
+        "all P": torch.full_like(good, P),
+        "random": torch.randint(0, P, good.shape, device="cuda", dtype=torch.int32, generator=g),
+        "beyond the arrays": good * 3,
+        "negative": -good,
+        "sawtooth": (good % 5000).contiguous(),
+    }
+    for label, row_ptr in wrong.items():
+        print("wrong row_ptr:", label, flush=True)
+        y = torch.full((rows + 64,), 3.0, dtype=torch.float16, device="cuda")
+        assert lib.macko_spmv_f16(c[0].data_ptr(), c[1].data_ptr(), row_ptr.data_ptr(), xg.data_ptr(), y.data_ptr(),
+                                  rows, cols, P, None) == 0
+        torch.cuda.synchronize()
+        assert bool((y[rows:] == 3.0).all())
+    y = macko_spmv.multiply((c[0], c[1], c[2].clone(), c[3], c[4]), xg)
+    helpers.assert_close_fp16(y.cpu().numpy(), helpers.dense_reference(dense, x))
